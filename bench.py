@@ -1,0 +1,146 @@
+#!/usr/bin/env python3
+"""Benchmark of the DM-block hot path on one MI355X.
+
+A "step" is one denoising step = one forward of the whole DiT stack over one synthetic joint sequence.
+Default workload: the full video DiT stack (28 blocks, d=4096, 32x128 heads, SwiGLU 16384, 512 text +
+16x44x80 video tokens = 56,832 tokens, bf16, random-init weights N(0, 0.02)).
+Prints ONE JSON line: ms per denoising step, the MFMA roofline of the dominant kernel (attention; duration
+from HIP events around every attention launch inside the timed region) and a CPU baseline (the fp32 oracle on
+this host's cores, bounded sample, extrapolated).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+
+def cpu_baseline(cfg, sample_tokens: int):
+    """fp32 oracle of ONE block on `sample_tokens` tokens of the same width, timed on the host cores; the GEMM
+    part scales linearly and the attention part quadratically with the token count."""
+    import torch
+    import oracle as O
+    d, h, H = cfg.d_model, cfg.hidden, cfg.n_heads
+    g = torch.Generator().manual_seed(0)
+    n = sample_tokens
+    x = torch.randn(n, d, generator=g)
+    w = dict(norm1_w=torch.ones(d), norm2_w=torch.ones(d))
+    for name, shape in (("wq", (d, d)), ("wk", (d, d)), ("wv", (d, d)), ("wo", (d, d)), ("wg", (h, d)), ("wu", (h, d)),
+                        ("wd", (d, h))):
+        w[name] = torch.randn(shape, generator=g) * 0.02
+    mod = [torch.randn(d, generator=g) * 0.1 for _ in range(6)]
+    pos = O.text_positions(0, n)
+    cos, sin = O.mrope_cos_sin(pos, cfg.head_dim, cfg.mrope_sections)
+    q = torch.randn(n, H, cfg.head_dim, generator=g)
+    def best_of_two(fn):
+        best = float("inf")
+        for _ in range(2):          # the first call of a size pays allocator growth / page faults
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+        return best
+    t_attn = best_of_two(lambda: O.attention(q, q, q))
+    t_block = best_of_two(lambda: O.dm_block(x, [w], mod, cos, sin, H))
+    t_lin = max(t_block - t_attn, 0.0)
+    ratio = cfg.n_tokens / n
+    per_block = t_lin * ratio + t_attn * ratio * ratio
+    return {"value": round(per_block * max(cfg.n_blocks, 1) * 1e3, 1), "unit": "ms per denoising step (extrapolated)",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"fp32 oracle, one block on {n} of {cfg.n_tokens} tokens at full width: {t_block:.2f} s "
+                      f"(attention {t_attn:.2f} s); linear part x{ratio:.2f}, attention x{ratio * ratio:.1f}, "
+                      f"x{max(cfg.n_blocks, 1)} blocks"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="C2", choices=["C0", "C2", "C3", "C4"])
+    ap.add_argument("--blocks", type=int, default=0, help="override the number of blocks (measurement aid; 0 = config)")
+    ap.add_argument("--attn-variant", type=int, default=0)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+
+    import dataclasses
+    import torch
+    from cosmos_amd import CONFIGS, DMStack, _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    cfg = CONFIGS[args.workload]
+    if args.blocks:
+        cfg = dataclasses.replace(cfg, n_blocks=args.blocks)
+    _lib.load()
+    ops.set_variant("attn", args.attn_variant)
+
+    stack = DMStack(cfg, device=dev)
+    stack.reset_parameters()
+    g = torch.Generator(device=dev).manual_seed(cfg.seed)
+    xv = torch.randn((1, cfg.n_video, cfg.d_model), generator=g, device=dev).to(torch.bfloat16)
+    xt = torch.randn((1, cfg.n_text, cfg.d_model), generator=g, device=dev).to(torch.bfloat16) if cfg.n_text else None
+    xa = torch.randn((1, cfg.n_action, cfg.d_model), generator=g, device=dev).to(torch.bfloat16) if cfg.n_action else None
+    t = torch.rand(1, generator=g, device=dev) * 1000.0
+
+    def step():
+        return stack(xv, t, encoder_hidden_states=xt, action_states=xa)[0]
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ops.time_attention(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    events = ops.time_attention(False)
+    assert bool(torch.isfinite(out.float()).all()), "non-finite output"
+
+    ms_per_step = wall * 1e3 / args.steps
+    attn_ms = [a.elapsed_time(b) for a, b in events]
+    attn_avg_ms = sum(attn_ms) / len(attn_ms)
+    attn_flops = cfg.attn_flops_per_block()
+    attn_tflops = attn_flops / (attn_avg_ms * 1e-3) / 1e12
+    gemm_ms_per_block = ms_per_step / cfg.n_blocks - attn_avg_ms     # everything that is not attention
+    gemm_tflops = cfg.gemm_flops_per_block() / (gemm_ms_per_block * 1e-3) / 1e12
+    peak = PEAK_BF16_TFLOPS
+    res = {
+        "metric": "ms per denoising step (DiT stack) on 1 GPU",
+        "value": round(ms_per_step, 2), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 2), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8-e4m3 GEMMs, bf16 attention" if cfg.fp8 else "bf16", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: {cfg.n_blocks} DM blocks, d={cfg.d_model}, {cfg.n_heads}x{cfg.head_dim} heads, "
+                               f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
+                               f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
+                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant},
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
+                     "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4), "traffic": None,
+                     "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},
+        "extra": {"ms_per_block": round(ms_per_step / cfg.n_blocks, 3),
+                  "non_attention_ms_per_block": round(gemm_ms_per_block, 3),
+                  "gemm_tflops_lower_bound": round(gemm_tflops, 1),
+                  "gemm_frac_of_peak_lower_bound": round(gemm_tflops / (PEAK_FP8_TFLOPS if cfg.fp8 else peak), 4),
+                  "total_tflops": round((attn_flops + cfg.gemm_flops_per_block()) * cfg.n_blocks / (ms_per_step * 1e-3) / 1e12, 1),
+                  "device": torch.cuda.get_device_name(0)},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,10 @@
+"""cosmos_amd - MI355X-native Cosmos 3 generator (DM) block forward.
+
+Python host code (PyTorch-ROCm for device memory and streams) over hand-written HIP kernels reached
+through the C ABI in include/cosmos_dm.h.
+"""
+from . import _lib, ops, rotary  # noqa: F401
+from .config import DMConfig, CONFIGS  # noqa: F401
+from .modules import DMAttention, DMAttnProcessor, DMBlock, DMStack, TimestepEmbedder, Workspace  # noqa: F401
+
+__version__ = "0.1.0"

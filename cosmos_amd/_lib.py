@@ -1,0 +1,74 @@
+"""ctypes binding of libcosmos_dm_hip.so (the C ABI declared in include/cosmos_dm.h).
+
+The product path has no CPU fallback: if the library is missing it is built once with hipcc, and if
+that fails, or a call returns a non-zero status, a RuntimeError is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+from . import build as _build
+
+_LOCK = threading.Lock()
+_LIB = None
+
+OK = 0
+ERR_BAD_ARG, ERR_BAD_SHAPE, ERR_BAD_ALIGN, ERR_NO_DEVICE, ERR_LAUNCH, ERR_UNSUPPORTED = -1, -2, -3, -4, -5, -6
+EPI_NONE, EPI_SWIGLU, EPI_GATE_RESIDUAL, EPI_ROPE_QK = 0, 1, 2, 3
+
+_P, _I64, _I32, _F32 = C.c_void_p, C.c_int64, C.c_int32, C.c_float
+
+# name -> (restype, argtypes); mirrors include/cosmos_dm.h one to one
+SIGNATURES = {
+    "cdm_version": (_I32, []),
+    "cdm_last_error": (C.c_char_p, []),
+    "cdm_device_count": (_I32, []),
+    "cdm_set_variant": (_I32, [C.c_char_p, _I32]),
+    "cdm_adaln_rmsnorm_bf16": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
+    "cdm_adaln_rmsnorm_quant_e4m3": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
+    "cdm_quant_rows_e4m3": (_I32, [_P, _I64, _P, _P, _I64, _I64, _P]),
+    "cdm_gemm_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P, _P, _P, _I64,
+                             _I32, _P]),
+    "cdm_gemm_fp8": (_I32, [_P, _I64, _P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P, _P,
+                            _P, _I64, _I32, _P]),
+    "cdm_mrope_qk_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I32, _I32, _P]),
+    "cdm_attn_workspace_bytes": (_I64, [_I64, _I32, _I32]),
+    "cdm_attn_fwd_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I32, _I32, _P, _I64, _P]),
+    "cdm_transpose_v_bf16": (_I32, [_P, _I64, _P, _I64, _I64, _I32, _I32, _P]),
+    "cdm_attn_fwd_vt_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _I32, _I32, _P]),
+    "cdm_grouped_gemm_bf16": (_I32, [_P, _I64, C.POINTER(_P), _I64, C.POINTER(_P), _P, _I64, C.POINTER(_I64),
+                                     C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P, _P, _I64,
+                                     _I32, _P]),
+}
+
+
+def lib_path() -> str:
+    return _build.LIB_PATH
+
+
+def load():
+    """Return the loaded library (building it first only if no built library exists)."""
+    global _LIB
+    with _LOCK:
+        if _LIB is not None:
+            return _LIB
+        path = lib_path()
+        if not os.path.exists(path):
+            _build.build(verbose=False)
+        lib = C.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)     # AttributeError here = the library does not export the ABI
+            fn.restype, fn.argtypes = res, args
+        _LIB = lib
+        return lib
+
+
+def last_error() -> str:
+    return load().cdm_last_error().decode("utf-8", "replace")
+
+
+def check(status: int, what: str) -> None:
+    if status != OK:
+        raise RuntimeError(f"{what} failed with status {status}: {last_error()}")

@@ -1,0 +1,408 @@
+// "NT" GEMM  C[M,N] = A[M,K] . W[N,K]^T  on the gfx950 matrix cores with fused epilogues, for bf16
+// operands (v_mfma_f32_32x32x16_bf16) and for e4m3 operands with per-row / per-column fp32 scales
+// (v_mfma_scale_f32_32x32x64_f8f6f4 with unit block scales; the rank-1 scale sa[i]*sw[j] is applied
+// to the fp32 accumulator in the epilogue).  A k-tile is 128 BYTES of K for both types, so the LDS
+// geometry, loads and swizzle are shared.
+//
+// Tiling: one workgroup (4 waves, 2x2) computes a 256x256 tile with BK = 64; each wave owns a
+// 128x128 sub-tile = 4x4 v_mfma_f32_32x32x16_bf16 accumulators (256 fp32 registers per lane).
+// Both operands are K-contiguous, so A and W fragments are plain 16-byte LDS reads.
+// Global -> LDS goes through the direct-to-LDS path (global_load_lds_dwordx4): each wave
+// instruction deposits 64 x 16 B = 8 tile rows linearly in LDS; bank conflicts are avoided by
+// permuting which 16-byte chunk of a row each lane fetches (XOR swizzle on the source side).
+// Two LDS stages (2 x 64 KB): the loads of k-tile t+1 are in flight while k-tile t is multiplied.
+// Workgroup ids are remapped so that each XCD (ids are dealt round-robin over the 8 XCDs) works
+// on a compact block of tiles and its private L2 sees the reuse.
+#include "cdm_common.h"
+
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kThreads = 256;
+constexpr int kTileBytes = BM * BK * 2;   // 32 KB per operand per stage
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+struct GemmParams {
+    const void* A; int64_t lda;          // operand strides in BYTES
+    const void* W; const void* W2; int64_t ldw;
+    const float* sa; const float* sw; const float* sw2;   // fp8 only
+    bf16_t* C; int64_t ldc;
+    int M, N, K;
+    const bf16_t* R; int64_t ldr;
+    const float* gate;
+    const float* cos; const float* sin;
+    int rope_cols, head_dim;
+    int tiles_m, tiles_n;
+};
+
+// chunk swizzle: 16-byte chunk c of tile row r lives at chunk position c ^ swz(r)
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+__device__ __forceinline__ bf16x8 lds_frag(const char* tile, int row, int chunk) {
+    return *reinterpret_cast<const bf16x8*>(tile + row * (BK * 2) + ((chunk ^ swz(row)) << 4));
+}
+
+template <bool FP8>
+__device__ __forceinline__ void compute_stage(const char* sa, const char* sb, f32x16 (&acc)[4][4], int wm, int wn,
+                                              int lane) {
+    const int r32 = lane & 31, kh = lane >> 5;
+    if (!FP8) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {     // 4 x 16 bf16 = 64 elements = 128 bytes
+            bf16x8 af[4], bfr[4];
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) af[mi] = lds_frag(sa, wm * 128 + mi * 32 + r32, 2 * ks + kh);
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) bfr[ni] = lds_frag(sb, wn * 128 + ni * 32 + r32, 2 * ks + kh);
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 4; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0);
+        }
+    } else {
+        // 2 x 64 e4m3: a lane supplies 32 consecutive bytes of K (two 16-byte chunks).  The same
+        // bytes go into the same operand slots for A and W, which is all the contraction needs.
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            i32x8 af[4], bfr[4];
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) {
+                const bf16x8 lo = lds_frag(sa, wm * 128 + mi * 32 + r32, 4 * ks + 2 * kh);
+                const bf16x8 hi = lds_frag(sa, wm * 128 + mi * 32 + r32, 4 * ks + 2 * kh + 1);
+                const int4 l4 = __builtin_bit_cast(int4, lo), h4 = __builtin_bit_cast(int4, hi);
+                af[mi] = i32x8{l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
+            }
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) {
+                const bf16x8 lo = lds_frag(sb, wn * 128 + ni * 32 + r32, 4 * ks + 2 * kh);
+                const bf16x8 hi = lds_frag(sb, wn * 128 + ni * 32 + r32, 4 * ks + 2 * kh + 1);
+                const int4 l4 = __builtin_bit_cast(int4, lo), h4 = __builtin_bit_cast(int4, hi);
+                bfr[ni] = i32x8{l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
+            }
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 4; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        af[mi], bfr[ni], acc[mi][ni], 0 /*A: e4m3*/, 0 /*B: e4m3*/, 0, 0x7f7f7f7f /*2^0*/, 0,
+                        0x7f7f7f7f);
+        }
+    }
+}
+
+// 8 + 8 direct-to-LDS loads of one k-tile: uniform base pointer (SGPR pair) + per-lane 32-bit byte offset
+__device__ __forceinline__ void issue_loads(const char* abase, const char* wbase, const char* w2base,
+                                            const uint32_t (&oa)[8], const uint32_t (&ob)[8], uint32_t w2mask,
+                                            char* sa, char* sb, int wave) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_global_load_lds(abase + oa[i], (lds_void*)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
+        const char* wb = ((w2mask >> i) & 1u) ? w2base : wbase;   // wave-uniform choice
+        __builtin_amdgcn_global_load_lds(wb + ob[i], (lds_void*)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+    }
+}
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
+
+template <int EPI, bool FP8>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(1024))) char sa0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char sb0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char sa1[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char sb1[kTileBytes];
+
+    // ---- XCD-aware tile assignment
+    const int total = p.tiles_m * p.tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    constexpr int GM = 8;
+    const int group = logical / (GM * p.tiles_n);
+    const int first_m = group * GM;
+    const int gsz = (p.tiles_m - first_m) < GM ? (p.tiles_m - first_m) : GM;
+    const int in_group = logical - group * GM * p.tiles_n;
+    const int tm = first_m + in_group % gsz;
+    const int tn = in_group / gsz;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = tm * BM;
+    const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
+
+    // ---- per-lane byte offsets (relative to the tile's first row) of the 8 + 8 loads of one k-tile
+    uint32_t oa[8], ob[8];
+    uint32_t w2mask = 0;     // bit i set: load i of this wave reads W2 (up_proj rows of a SWIGLU tile)
+    int nb0 = n0;            // first W row of the tile
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = (i * 4 + wave) * 8 + (lane >> 3);   // tile row this lane feeds
+        const int chunk = (lane & 7) ^ swz(row);            // source chunk that belongs at position lane&7
+        int am = row;
+        am = (m0 + am) < p.M ? am : p.M - 1 - m0;
+        oa[i] = (uint32_t)(am * (int)p.lda + chunk * 16);
+        int bn;
+        if (EPI == CDM_EPI_SWIGLU) {
+            // 64-row groups of the tile alternate gate / up: [g 0-63 | u 0-63 | g 64-127 | u 64-127]
+            const int grp = ((i * 4 + wave) * 8) >> 6;       // wave-uniform
+            if (grp & 1) w2mask |= 1u << i;
+            bn = (grp >> 1) * 64 + (row & 63);
+        } else {
+            bn = row;
+        }
+        bn = (nb0 + bn) < p.N ? bn : p.N - 1 - nb0;
+        ob[i] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
+    }
+    const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
+    const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)nb0 * p.ldw;
+    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)nb0 * p.ldw : wbase;
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+    const int KT = p.K / (FP8 ? 128 : 64);   // k-tiles of 128 bytes; the host guarantees an even count
+    issue_loads(abase, wbase, w2base, oa, ob, w2mask, sa0, sb0, wave);
+    for (int kt = 0; kt < KT; kt += 2) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        issue_loads(abase + (kt + 1) * 128, wbase + (kt + 1) * 128, w2base + (kt + 1) * 128, oa, ob, w2mask, sa1, sb1,
+                    wave);
+        __builtin_amdgcn_sched_barrier(0);      // keep the prefetch at the top of the stage
+        compute_stage<FP8>(sa0, sb0, acc, wm, wn, lane);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (kt + 2 < KT)
+            issue_loads(abase + (kt + 2) * 128, wbase + (kt + 2) * 128, w2base + (kt + 2) * 128, oa, ob, w2mask, sa0,
+                        sb0, wave);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_stage<FP8>(sa1, sb1, acc, wm, wn, lane);
+    }
+
+    // ---- epilogue: accumulator (mi, ni, v) is row 8*(v/4) + 4*(lane/32) + v%4, column lane%32 of its 32x32 block
+    const int r32 = lane & 31, kh = lane >> 5;
+    const int row_base = m0 + wm * 128 + 4 * kh;
+    if (EPI == CDM_EPI_SWIGLU) {
+        const int col_base = n0 + wn * 64 + r32;      // wave's 128 tile columns = [gate 64 | up 64]
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int nj = 0; nj < 2; ++nj) {
+                const int col = col_base + nj * 32;
+                if (col >= p.N) continue;
+                float sg = 1.0f, su = 1.0f;
+                if (FP8) { sg = p.sw[col]; su = p.sw2[col]; }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
+                    if (row < p.M) {
+                        float g = acc[mi][nj][v], u = acc[mi][nj + 2][v];
+                        if (FP8) { const float sr = p.sa[row]; g *= sr * sg; u *= sr * su; }
+                        p.C[(int64_t)row * p.ldc + col] = __builtin_bit_cast(bf16_t, (__bf16)(silu_f(g) * u));
+                    }
+                }
+            }
+        return;
+    }
+    const int col_base = n0 + wn * 128 + r32;
+    if (FP8) {      // rank-1 dequantisation scale on the fp32 accumulators
+        float sc[4];
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) { const int col = col_base + ni * 32; sc[ni] = col < p.N ? p.sw[col] : 0.0f; }
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
+                const float sr = p.sa[row < p.M ? row : p.M - 1];
+#pragma unroll
+                for (int ni = 0; ni < 4; ++ni) acc[mi][ni][v] *= sr * sc[ni];
+            }
+    }
+    if (EPI == CDM_EPI_ROPE_QK) {
+        if (n0 + wn * 128 < p.rope_cols) {     // wave-uniform: this wave's 128 columns are whole heads of Q or K
+            const int half = p.head_dim >> 1;
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
+                    const int rr = row < p.M ? row : p.M - 1;
+                    if (p.head_dim == 128) {
+#pragma unroll
+                        for (int nj = 0; nj < 2; ++nj) {
+                            const int i = nj * 32 + r32;
+                            const float c = p.cos[(int64_t)rr * half + i], s = p.sin[(int64_t)rr * half + i];
+                            const float x1 = acc[mi][nj][v], x2 = acc[mi][nj + 2][v];
+                            acc[mi][nj][v] = x1 * c - x2 * s;
+                            acc[mi][nj + 2][v] = x2 * c + x1 * s;
+                        }
+                    } else {   // head_dim 64: two heads per wave, pairs are adjacent 32-column blocks
+                        const float c = p.cos[(int64_t)rr * half + r32], s = p.sin[(int64_t)rr * half + r32];
+#pragma unroll
+                        for (int nj = 0; nj < 4; nj += 2) {
+                            const float x1 = acc[mi][nj][v], x2 = acc[mi][nj + 1][v];
+                            acc[mi][nj][v] = x1 * c - x2 * s;
+                            acc[mi][nj + 1][v] = x2 * c + x1 * s;
+                        }
+                    }
+                }
+        }
+    }
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) {
+            const int col = col_base + ni * 32;
+            if (col >= p.N) continue;
+            float gt = 1.0f;
+            if (EPI == CDM_EPI_GATE_RESIDUAL && p.gate) gt = p.gate[col];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
+                if (row < p.M) {
+                    float val = acc[mi][ni][v];
+                    if (EPI == CDM_EPI_GATE_RESIDUAL) {
+                        const float res = bf16_bits_to_f32(p.R[(int64_t)row * p.ldr + col]);
+                        val = res + gt * val;
+                    }
+                    p.C[(int64_t)row * p.ldc + col] = __builtin_bit_cast(bf16_t, (__bf16)val);
+                }
+            }
+        }
+}
+
+// esize = bytes per operand element (2 = bf16, 1 = e4m3); strides in elements
+int32_t validate(const char* who, int esize, const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2,
+                 void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epi, const void* R, int64_t ldr,
+                 const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim) {
+    const int64_t kmult = 256 / esize;      // two 128-byte k-tiles
+    CDM_REQUIRE(A && W && C, CDM_ERR_BAD_ARG, "%s: null pointer", who);
+    CDM_REQUIRE(M >= 0 && N > 0 && K > 0, CDM_ERR_BAD_ARG, "%s: bad sizes M=%lld N=%lld K=%lld", who, (long long)M,
+                (long long)N, (long long)K);
+    CDM_REQUIRE(epi >= CDM_EPI_NONE && epi <= CDM_EPI_ROPE_QK, CDM_ERR_BAD_ARG, "%s: unknown epilogue %d", who, epi);
+    CDM_REQUIRE(K % kmult == 0, CDM_ERR_BAD_SHAPE, "%s: K=%lld must be a multiple of %lld", who, (long long)K,
+                (long long)kmult);
+    CDM_REQUIRE(N % 8 == 0, CDM_ERR_BAD_SHAPE, "%s: N=%lld must be a multiple of 8", who, (long long)N);
+    CDM_REQUIRE(M < (1ll << 31) - 512 && N < (1ll << 31) - 512 && K < (1ll << 24) && lda < (1ll << 22) &&
+                    ldw < (1ll << 22),
+                CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
+    CDM_REQUIRE(lda >= K && ldw >= K && ldc >= N, CDM_ERR_BAD_ARG, "%s: row stride smaller than row length", who);
+    CDM_REQUIRE(cdm_aligned16(A) && cdm_aligned16(W) && cdm_aligned16(C) && (lda * esize) % 16 == 0 &&
+                    (ldw * esize) % 16 == 0,
+                CDM_ERR_BAD_ALIGN, "%s: pointers/strides must be 16-byte aligned", who);
+    if (epi == CDM_EPI_SWIGLU)
+        CDM_REQUIRE(W2 && cdm_aligned16(W2), CDM_ERR_BAD_ARG, "%s: SWIGLU needs an aligned W2 (up_proj)", who);
+    if (epi == CDM_EPI_GATE_RESIDUAL)
+        CDM_REQUIRE(R && ldr >= N, CDM_ERR_BAD_ARG, "%s: GATE_RESIDUAL needs R with ldr >= N", who);
+    if (epi == CDM_EPI_ROPE_QK) {
+        CDM_REQUIRE(cos && sin, CDM_ERR_BAD_ARG, "%s: ROPE_QK needs cos/sin tables", who);
+        CDM_REQUIRE(head_dim == 64 || head_dim == 128, CDM_ERR_BAD_SHAPE, "%s: head_dim=%d must be 64 or 128", who,
+                    head_dim);
+        CDM_REQUIRE(rope_cols >= 0 && rope_cols <= N && rope_cols % 256 == 0, CDM_ERR_BAD_SHAPE,
+                    "%s: rope_cols=%lld must be a multiple of 256 within N", who, (long long)rope_cols);
+    }
+    return CDM_OK;
+}
+
+template <bool FP8>
+int32_t run(GemmParams& p, int64_t M, int64_t N, int32_t epilogue, hipStream_t st, const char* who) {
+    p.tiles_m = (int)((M + BM - 1) / BM);
+    const int tile_n = epilogue == CDM_EPI_SWIGLU ? BN / 2 : BN;
+    p.tiles_n = (int)((N + tile_n - 1) / tile_n);
+    const int total = p.tiles_m * p.tiles_n;
+    const int grid = ((total + 7) / 8) * 8;
+    switch (epilogue) {
+        case CDM_EPI_NONE: gemm_kernel<CDM_EPI_NONE, FP8><<<grid, kThreads, 0, st>>>(p); break;
+        case CDM_EPI_SWIGLU: gemm_kernel<CDM_EPI_SWIGLU, FP8><<<grid, kThreads, 0, st>>>(p); break;
+        case CDM_EPI_GATE_RESIDUAL: gemm_kernel<CDM_EPI_GATE_RESIDUAL, FP8><<<grid, kThreads, 0, st>>>(p); break;
+        default: gemm_kernel<CDM_EPI_ROPE_QK, FP8><<<grid, kThreads, 0, st>>>(p); break;
+    }
+    return cdm_check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2, void* C,
+                                 int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epilogue, const void* R,
+                                 int64_t ldr, const float* gate, const float* cos, const float* sin,
+                                 int64_t rope_cols, int32_t head_dim, void* stream) {
+    int32_t rc = validate("gemm_bf16", 2, A, lda, W, ldw, W2, C, ldc, M, N, K, epilogue, R, ldr, cos, sin, rope_cols,
+                          head_dim);
+    if (rc) return rc;
+    if ((rc = cdm_require_device())) return rc;
+    if (M == 0) return CDM_OK;
+    GemmParams p{};
+    p.A = A; p.lda = lda * 2;
+    p.W = W; p.W2 = W2; p.ldw = ldw * 2;
+    p.C = (bf16_t*)C; p.ldc = ldc;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.R = (const bf16_t*)R; p.ldr = ldr; p.gate = gate;
+    p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
+    return run<false>(p, M, N, epilogue, (hipStream_t)stream, "gemm_bf16");
+}
+
+extern "C" int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const void* Wq, int64_t ldw,
+                                const float* sw, const void* W2q, const float* sw2, void* C, int64_t ldc, int64_t M,
+                                int64_t N, int64_t K, int32_t epilogue, const void* R, int64_t ldr, const float* gate,
+                                const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
+                                void* stream) {
+    int32_t rc = validate("gemm_fp8", 1, Aq, lda, Wq, ldw, W2q, C, ldc, M, N, K, epilogue, R, ldr, cos, sin, rope_cols,
+                          head_dim);
+    if (rc) return rc;
+    CDM_REQUIRE(sa && sw, CDM_ERR_BAD_ARG, "gemm_fp8: null scale pointer");
+    if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(sw2, CDM_ERR_BAD_ARG, "gemm_fp8: SWIGLU needs sw2");
+    if ((rc = cdm_require_device())) return rc;
+    if (M == 0) return CDM_OK;
+    GemmParams p{};
+    p.A = Aq; p.lda = lda;
+    p.W = Wq; p.W2 = W2q; p.ldw = ldw;
+    p.sa = sa; p.sw = sw; p.sw2 = sw2;
+    p.C = (bf16_t*)C; p.ldc = ldc;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.R = (const bf16_t*)R; p.ldr = ldr; p.gate = gate;
+    p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
+    return run<true>(p, M, N, epilogue, (hipStream_t)stream, "gemm_fp8");
+}
+
+extern "C" int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw,
+                                         const void* const* W2, void* C, int64_t ldc, const int64_t* seg_start,
+                                         const int64_t* seg_len, int32_t n_seg, int64_t N, int64_t K,
+                                         int32_t epilogue, const void* R, int64_t ldr, const float* const* gate,
+                                         const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
+                                         void* stream) {
+    CDM_REQUIRE(A && W && C && seg_start && seg_len, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: null pointer");
+    CDM_REQUIRE(n_seg >= 0 && n_seg <= 64, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: n_seg=%d out of range", n_seg);
+    if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(W2, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: SWIGLU needs W2");
+    // validate every segment before anything is enqueued
+    for (int g = 0; g < n_seg; ++g) {
+        CDM_REQUIRE(seg_start[g] >= 0 && seg_len[g] >= 0, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: negative segment");
+        CDM_REQUIRE(W[g], CDM_ERR_BAD_ARG, "grouped_gemm_bf16: null weight for segment %d", g);
+        CDM_REQUIRE((seg_start[g] * lda) % 8 == 0 && (seg_start[g] * ldc) % 8 == 0, CDM_ERR_BAD_ALIGN,
+                    "grouped_gemm_bf16: segment %d does not start on a 16-byte boundary", g);
+        const bf16_t* a = (const bf16_t*)A + seg_start[g] * lda;
+        int32_t rc = validate("grouped_gemm_bf16", 2, a, lda, W[g], ldw, W2 ? W2[g] : nullptr,
+                              (bf16_t*)C + seg_start[g] * ldc, ldc, seg_len[g], N, K, epilogue,
+                              R ? (const bf16_t*)R + seg_start[g] * ldr : nullptr, ldr, cos, sin, rope_cols, head_dim);
+        if (rc) return rc;
+    }
+    for (int g = 0; g < n_seg; ++g) {
+        const int64_t s0 = seg_start[g];
+        const int half = head_dim / 2;
+        int32_t rc = cdm_gemm_bf16((const bf16_t*)A + s0 * lda, lda, W[g], ldw, W2 ? W2[g] : nullptr,
+                                   (bf16_t*)C + s0 * ldc, ldc, seg_len[g], N, K, epilogue,
+                                   R ? (const bf16_t*)R + s0 * ldr : nullptr, ldr, gate ? gate[g] : nullptr,
+                                   cos ? cos + s0 * half : nullptr, sin ? sin + s0 * half : nullptr, rope_cols,
+                                   head_dim, stream);
+        if (rc) return rc;
+    }
+    return CDM_OK;
+}

@@ -1,0 +1,359 @@
+"""Diffusers-style host side of the Cosmos 3 generator (DM) block: transformer stack -> block ->
+attention module -> pluggable attention processor, all of whose tensor work runs in the HIP library.
+
+Calling idiom mirrored (NVIDIA/cosmos README.md:238-263 drives it through the diffusers pipeline):
+    stack(hidden_states, timestep, encoder_hidden_states) -> for block in blocks: block(...)
+    block: per-branch adaLN-RMSNorm -> attn.processor(attn, ...) -> gated residual ->
+           per-branch adaLN-RMSNorm -> per-branch SwiGLU -> gated residual          (README.md:74)
+Per-branch ("Mixture-of-Transformers") weights: branch b of a layer owns
+    attn.qkv_weight[b]  rows [0,d) | [d,2d) | [2d,3d) = add_q_proj | add_k_proj | add_v_proj (DM) or to_q | to_k | to_v (AR)
+    attn.out_weight[b]  = to_add_out (DM) / to_out (AR)
+    norm1_weight[b], norm2_weight[b], gate_weight[b], up_weight[b], down_weight[b] = the branch's norms and MLP
+(parameter names as in transformers models/cosmos3_omni/modeling_cosmos3_omni.py:39-60).
+Only timestep conditioning (a one-row MLP) is left to torch ops.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+from torch import nn
+
+from . import ops, rotary
+from .config import DMConfig
+
+Segment = rotary.Segment
+
+
+def _as2d(t: torch.Tensor) -> torch.Tensor:
+    if t.dim() == 3:
+        if t.shape[0] != 1:
+            raise NotImplementedError("batch size must be 1 (one joint sequence per forward)")
+        return t[0]
+    return t
+
+
+class Workspace:
+    """Caller-owned scratch tensors of one (n_tokens, d, hidden) shape, reused by every block."""
+
+    def __init__(self, n: int, d: int, hidden: int, n_heads: int, head_dim: int, device):
+        bf = dict(dtype=torch.bfloat16, device=device)
+        self.n, self.d, self.hidden = n, d, hidden
+        self.y = torch.empty((n, d), **bf)
+        self.qkv = torch.empty((n, 3 * d), **bf)
+        self.attn_out = torch.empty((n, d), **bf)
+        self.h = torch.empty((n, hidden), **bf)
+        self.attn_ws = torch.empty((max(ops.attn_workspace_bytes(n, n_heads, head_dim), 16),), dtype=torch.uint8,
+                                   device=device)
+
+    def fits(self, n: int, d: int, hidden: int) -> bool:
+        return (self.n, self.d, self.hidden) == (n, d, hidden)
+
+
+class DMAttnProcessor:
+    """Attention processor: per-branch QKV projection with mRoPE in the GEMM epilogue, ONE shared full
+    attention over the joint sequence, per-branch output projection (optionally fused with the gated
+    residual)."""
+
+    def __call__(self, attn: "DMAttention", hidden_states: torch.Tensor,
+                 encoder_hidden_states: Optional[torch.Tensor] = None, attention_mask: Optional[torch.Tensor] = None,
+                 image_rotary_emb: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, *,
+                 modality_segments: Optional[Sequence[Segment]] = None, residual: Optional[torch.Tensor] = None,
+                 gate: Optional[torch.Tensor] = None, quant_scale: Optional[torch.Tensor] = None,
+                 workspace: Optional[Workspace] = None):
+        if attention_mask is not None:
+            raise NotImplementedError("the DM branch uses full attention; attention_mask must be None")
+        if image_rotary_emb is None:
+            raise ValueError("image_rotary_emb=(cos, sin) is required")
+        batched = hidden_states.dim() == 3
+        x = _as2d(hidden_states)
+        n_enc = 0
+        if encoder_hidden_states is not None:
+            # diffusers joint-attention convention: context tokens first, then the latent tokens
+            if quant_scale is not None or residual is not None:
+                raise NotImplementedError("encoder_hidden_states cannot be combined with fused residual / fp8 input")
+            enc = _as2d(encoder_hidden_states)
+            n_enc = enc.shape[0]
+            x = torch.cat([enc, x], dim=0)
+            if modality_segments is None:
+                dm = min(1, attn.n_branches - 1)      # branch 0 serves the context tokens
+                modality_segments = [(0, n_enc, 0, False), (n_enc, x.shape[0] - n_enc, dm, True)]
+        n, d = x.shape[0], attn.d_model
+        if modality_segments is None:
+            modality_segments = [(0, n, 0, True)]
+        cos, sin = image_rotary_emb
+        ws = workspace
+        qkv = ws.qkv if ws is not None else torch.empty((n, 3 * d), dtype=torch.bfloat16, device=x.device)
+        o = ws.attn_out if ws is not None else torch.empty((n, d), dtype=torch.bfloat16, device=x.device)
+
+        attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
+                     rope_cols=2 * d, head_dim=attn.head_dim)
+        ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], attn.n_heads, attn.head_dim, out=o,
+                      workspace=ws.attn_ws if ws is not None else None)
+        if attn.fp8:
+            oq, so = ops.quant_rows(o)
+        else:
+            oq, so = o, None
+        if residual is not None:
+            res = _as2d(residual)
+            gates = [gate if modulated else None for (_, _, _, modulated) in modality_segments]
+            attn._linear(oq, so, "out", modality_segments, out=res, epilogue="gate_residual", residual=res,
+                         gates=gates)
+            return residual
+        out = torch.empty((n, d), dtype=torch.bfloat16, device=x.device)
+        attn._linear(oq, so, "out", modality_segments, out=out, epilogue="none")
+        if encoder_hidden_states is not None:
+            h, e = out[n_enc:], out[:n_enc]
+            return (h.unsqueeze(0), e.unsqueeze(0)) if batched else (h, e)
+        return out.unsqueeze(0) if batched else out
+
+
+class DMAttention(nn.Module):
+    """Attention module of one MoT layer: per-branch projections around one shared attention."""
+
+    def __init__(self, d_model: int, n_heads: int, head_dim: int, n_branches: int = 1, fp8: bool = False,
+                 processor: Optional[DMAttnProcessor] = None, device=None, dtype=torch.bfloat16):
+        super().__init__()
+        if n_heads * head_dim != d_model:
+            raise ValueError("n_heads * head_dim must equal d_model")
+        self.d_model, self.n_heads, self.head_dim, self.n_branches, self.fp8 = d_model, n_heads, head_dim, n_branches, fp8
+        kw = dict(device=device, dtype=dtype)
+        self.qkv_weight = nn.ParameterList([nn.Parameter(torch.empty(3 * d_model, d_model, **kw), requires_grad=False)
+                                            for _ in range(n_branches)])
+        self.out_weight = nn.ParameterList([nn.Parameter(torch.empty(d_model, d_model, **kw), requires_grad=False)
+                                            for _ in range(n_branches)])
+        self.processor = processor or DMAttnProcessor()
+        self._q = {}     # fp8 copies: name -> list of (wq, sw)
+
+    def set_processor(self, processor) -> None:
+        self.processor = processor
+
+    def quantize_(self) -> None:
+        """Offline per-output-channel e4m3 quantisation of this module's weights (fp8 variant)."""
+        self._q["qkv"] = [ops.quant_rows(w.data) for w in self.qkv_weight]
+        self._q["out"] = [ops.quant_rows(w.data) for w in self.out_weight]
+
+    def _weights(self, which: str):
+        return self.qkv_weight if which == "qkv" else self.out_weight
+
+    def _linear(self, a: torch.Tensor, sa: Optional[torch.Tensor], which: str, segments: Sequence[Segment], *,
+                out: torch.Tensor, epilogue: str, residual=None, gates=None, cos=None, sin=None, rope_cols=0,
+                head_dim=0) -> None:
+        _routed_linear(a, sa, self._weights(which), self._q.get(which) if self.fp8 else None, None, segments, out=out,
+                       epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
+                       head_dim=head_dim)
+
+    def forward(self, hidden_states, encoder_hidden_states=None, attention_mask=None, image_rotary_emb=None, **kw):
+        return self.processor(self, hidden_states, encoder_hidden_states=encoder_hidden_states,
+                              attention_mask=attention_mask, image_rotary_emb=image_rotary_emb, **kw)
+
+
+def _routed_linear(a, sa, weights, qweights, weights2, segments, *, out, epilogue, residual=None, gates=None, cos=None,
+                   sin=None, rope_cols=0, head_dim=0, qweights2=None) -> None:
+    """Per-modality linear over contiguous token segments (one kernel launch per segment)."""
+    if qweights is None and len(segments) > 1:
+        ops.grouped_gemm(a, [weights[b] for (_, _, b, _) in segments], [(s, l) for (s, l, _, _) in segments],
+                         w2s=[weights2[b] for (_, _, b, _) in segments] if weights2 is not None else None,
+                         epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
+                         head_dim=head_dim, out=out)
+        return
+    for i, (s0, ln, b, _) in enumerate(segments):
+        sl = slice(s0, s0 + ln)
+        kw = dict(epilogue=epilogue, residual=residual[sl] if residual is not None else None,
+                  gate=gates[i] if gates is not None else None, cos=cos[sl] if cos is not None else None,
+                  sin=sin[sl] if sin is not None else None, rope_cols=rope_cols, head_dim=head_dim, out=out[sl])
+        if qweights is not None:
+            wq, sw = qweights[b]
+            w2q, sw2 = qweights2[b] if qweights2 is not None else (None, None)
+            ops.gemm_fp8(a[sl], sa[sl], wq, sw, w2q=w2q, sw2=sw2, **kw)
+        else:
+            ops.gemm(a[sl], weights[b], w2=weights2[b] if weights2 is not None else None, **kw)
+
+
+class DMBlock(nn.Module):
+    """One Mixture-of-Transformers layer (generator side)."""
+
+    def __init__(self, d_model: int, n_heads: int, head_dim: int, hidden: int, n_branches: int = 1,
+                 eps: float = 1e-6, fp8: bool = False, device=None, dtype=torch.bfloat16):
+        super().__init__()
+        kw = dict(device=device, dtype=dtype)
+        self.d_model, self.hidden, self.eps, self.fp8, self.n_branches = d_model, hidden, eps, fp8, n_branches
+        self.attn = DMAttention(d_model, n_heads, head_dim, n_branches, fp8, device=device, dtype=dtype)
+        P = lambda *shape: nn.Parameter(torch.empty(*shape, **kw), requires_grad=False)
+        self.norm1_weight = nn.ParameterList([P(d_model) for _ in range(n_branches)])
+        self.norm2_weight = nn.ParameterList([P(d_model) for _ in range(n_branches)])
+        self.gate_weight = nn.ParameterList([P(hidden, d_model) for _ in range(n_branches)])
+        self.up_weight = nn.ParameterList([P(hidden, d_model) for _ in range(n_branches)])
+        self.down_weight = nn.ParameterList([P(d_model, hidden) for _ in range(n_branches)])
+        self.adaLN_modulation = nn.Linear(d_model, 6 * d_model, bias=True, **kw)
+        self._q = {}
+        self._ws: Optional[Workspace] = None
+
+    @torch.no_grad()
+    def reset_parameters(self, generator: Optional[torch.Generator] = None, std: float = 0.02) -> None:
+        for name, p in self.named_parameters():
+            if "norm" in name:
+                p.fill_(1.0)
+            elif name.endswith("bias"):
+                p.zero_()
+            else:
+                p.copy_((torch.randn(p.shape, generator=generator, device=p.device, dtype=torch.float32) * std).to(p.dtype))
+        if self.fp8:
+            self.quantize_()
+
+    def quantize_(self) -> None:
+        self.attn.quantize_()
+        for name, plist in (("gate", self.gate_weight), ("up", self.up_weight), ("down", self.down_weight)):
+            self._q[name] = [ops.quant_rows(w.data) for w in plist]
+
+    def modulation(self, temb: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+        """(shift1, scale1, gate1, shift2, scale2, gate2), each [d] fp32, from the conditioning vector."""
+        c = temb.reshape(1, -1).to(self.adaLN_modulation.weight.dtype)
+        m = self.adaLN_modulation(torch.nn.functional.silu(c)).float().reshape(-1)
+        return tuple(t.contiguous() for t in m.chunk(6))
+
+    def _norm(self, x, weights, shift, scale, segments, y):
+        """Per-branch adaLN-RMSNorm into y (bf16), or into fresh (e4m3, scale) tensors for the fp8 variant."""
+        if not self.fp8:
+            for (s0, ln, b, modulated) in segments:
+                ops.adaln_rmsnorm(x[s0:s0 + ln], weights[b], shift if modulated else None, scale if modulated else None,
+                                  self.eps, out=y[s0:s0 + ln])
+            return y, None
+        yq = torch.empty(x.shape, dtype=ops.FP8_DTYPE, device=x.device)
+        st = torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)
+        for (s0, ln, b, modulated) in segments:
+            q, s = ops.adaln_rmsnorm_quant(x[s0:s0 + ln], weights[b], shift if modulated else None,
+                                           scale if modulated else None, self.eps)
+            yq[s0:s0 + ln].copy_(q); st[s0:s0 + ln].copy_(s)
+        return yq, st
+
+    def forward(self, hidden_states: torch.Tensor, temb: torch.Tensor,
+                image_rotary_emb: Tuple[torch.Tensor, torch.Tensor],
+                modality_segments: Optional[Sequence[Segment]] = None, *, inplace: bool = False,
+                modulation: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[Workspace] = None):
+        batched = hidden_states.dim() == 3
+        x = _as2d(hidden_states)
+        if not inplace:
+            x = x.clone()
+        n, d = x.shape
+        segs = list(modality_segments) if modality_segments is not None else [(0, n, 0, True)]
+        ws = workspace or self._ws
+        if ws is None or not ws.fits(n, d, self.hidden) or ws.y.device != x.device:
+            ws = Workspace(n, d, self.hidden, self.attn.n_heads, self.attn.head_dim, x.device)
+            if workspace is None:
+                self._ws = ws
+        sh1, sc1, g1, sh2, sc2, g2 = modulation if modulation is not None else self.modulation(temb)
+
+        y, sy = self._norm(x, self.norm1_weight, sh1, sc1, segs, ws.y)
+        self.attn(y, image_rotary_emb=image_rotary_emb, modality_segments=segs, residual=x, gate=g1, quant_scale=sy,
+                  workspace=ws)
+        y, sy = self._norm(x, self.norm2_weight, sh2, sc2, segs, ws.y)
+        q = self._q if self.fp8 else {}
+        _routed_linear(y, sy, self.gate_weight, q.get("gate"), self.up_weight, segs, out=ws.h, epilogue="swiglu",
+                       qweights2=q.get("up"))
+        if self.fp8:
+            hq, sh = ops.quant_rows(ws.h)
+        else:
+            hq, sh = ws.h, None
+        gates = [g2 if modulated else None for (_, _, _, modulated) in segs]
+        _routed_linear(hq, sh, self.down_weight, q.get("down"), None, segs, out=x, epilogue="gate_residual",
+                       residual=x, gates=gates)
+        return x.unsqueeze(0) if batched else x
+
+
+class TimestepEmbedder(nn.Module):
+    """256-d sinusoidal embedding of t -> Linear -> SiLU -> Linear (stays in torch: a one-row MLP)."""
+
+    def __init__(self, d_model: int, freq_dim: int = 256, device=None, dtype=torch.float32):
+        super().__init__()
+        self.freq_dim = freq_dim
+        self.linear_1 = nn.Linear(freq_dim, d_model, device=device, dtype=dtype)
+        self.linear_2 = nn.Linear(d_model, d_model, device=device, dtype=dtype)
+
+    def sinusoid(self, t: torch.Tensor) -> torch.Tensor:
+        half = self.freq_dim // 2
+        k = torch.arange(half, dtype=torch.float32, device=t.device)
+        f = torch.exp(-math.log(10000.0) * k / half)
+        a = t.to(torch.float32).reshape(-1, 1) * f.reshape(1, -1)
+        return torch.cat([a.cos(), a.sin()], dim=-1)
+
+    def forward(self, t: torch.Tensor) -> torch.Tensor:
+        e = self.sinusoid(t).to(self.linear_1.weight.dtype)
+        return self.linear_2(torch.nn.functional.silu(self.linear_1(e)))
+
+
+class DMStack(nn.Module):
+    """L blocks over the joint sequence text | video | action (diffusers transformer forward shape)."""
+
+    def __init__(self, cfg: DMConfig, device=None, dtype=torch.bfloat16):
+        super().__init__()
+        self.cfg = cfg
+        self.time_embedder = TimestepEmbedder(cfg.d_model, device=device)
+        self.blocks = nn.ModuleList([DMBlock(cfg.d_model, cfg.n_heads, cfg.head_dim, cfg.hidden, cfg.n_branches,
+                                             cfg.eps, cfg.fp8, device=device, dtype=dtype)
+                                     for _ in range(cfg.n_blocks)])
+        self._rot = None
+        self._ws: Optional[Workspace] = None
+
+    @torch.no_grad()
+    def reset_parameters(self, seed: Optional[int] = None) -> None:
+        dev = next(self.parameters()).device
+        g = torch.Generator(device=dev).manual_seed(self.cfg.seed if seed is None else seed)
+        for p in self.time_embedder.parameters():
+            if p.dim() == 2:
+                p.copy_(torch.randn(p.shape, generator=g, device=dev) * 0.02)
+            else:
+                p.zero_()
+        for b in self.blocks:
+            b.reset_parameters(g)
+
+    def segments(self) -> List[Segment]:
+        """(start, len, branch, modulated): text uses branch 0 un-modulated; video and action are modulated."""
+        c = self.cfg
+        multi = c.n_branches > 1
+        segs, s = [], 0
+        if c.n_text:
+            segs.append((s, c.n_text, 0, False)); s += c.n_text
+        segs.append((s, c.n_video, 1 if multi else 0, True)); s += c.n_video
+        if c.n_action:
+            segs.append((s, c.n_action, min(2, c.n_branches - 1), True))
+        return segs
+
+    def rotary(self, device) -> Tuple[torch.Tensor, torch.Tensor]:
+        if self._rot is None or self._rot[0].device != torch.device(device):
+            c = self.cfg
+            pos, _ = rotary.build_positions(c.n_text, c.grid, c.n_action)
+            self._rot = rotary.rotary_tables(pos, c.head_dim, c.mrope_sections, c.rope_base, c.rope_layout, device)
+        return self._rot
+
+    @torch.no_grad()
+    def forward(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
+                encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
+                return_dict: bool = False):
+        c = self.cfg
+        parts = []
+        if c.n_text:
+            if encoder_hidden_states is None:
+                raise ValueError("this configuration expects encoder_hidden_states (text context)")
+            parts.append(_as2d(encoder_hidden_states))
+        parts.append(_as2d(hidden_states))
+        if c.n_action:
+            if action_states is None:
+                raise ValueError("this configuration expects action_states")
+            parts.append(_as2d(action_states))
+        x = torch.cat(parts, dim=0).contiguous() if len(parts) > 1 else parts[0].clone()
+        if x.shape != (c.n_tokens, c.d_model):
+            raise ValueError(f"joint sequence has shape {tuple(x.shape)}, expected {(c.n_tokens, c.d_model)}")
+        rot = self.rotary(x.device)
+        segs = self.segments()
+        temb = self.time_embedder(timestep.reshape(-1)[:1])
+        if self._ws is None or not self._ws.fits(c.n_tokens, c.d_model, c.hidden) or self._ws.y.device != x.device:
+            self._ws = Workspace(c.n_tokens, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
+        for blk in self.blocks:
+            blk(x, temb, rot, segs, inplace=True, workspace=self._ws)
+        video = x[c.n_text:c.n_text + c.n_video]
+        out = video.unsqueeze(0) if hidden_states.dim() == 3 else video
+        if return_dict:
+            return {"sample": out, "joint": x}
+        return (out,)

@@ -1,0 +1,243 @@
+"""Thin torch-tensor wrappers over the C ABI (include/cosmos_dm.h).
+
+Each function validates what the C side cannot see (dtype, device, innermost stride), then passes raw
+device pointers, sizes, row strides and the current HIP stream.  There is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import EPI_GATE_RESIDUAL, EPI_NONE, EPI_ROPE_QK, EPI_SWIGLU
+
+_EPI = {"none": EPI_NONE, "swiglu": EPI_SWIGLU, "gate_residual": EPI_GATE_RESIDUAL, "rope_qk": EPI_ROPE_QK}
+FP8_DTYPE = torch.float8_e4m3fn
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _chk(t: Optional[torch.Tensor], name: str, dtype=None, ndim: Optional[int] = None) -> int:
+    if t is None:
+        return 0
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (the HIP path has no CPU fallback)")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError(f"{name} must be {ndim}-D, got shape {tuple(t.shape)}")
+    if t.dim() and t.stride(-1) != 1:
+        raise ValueError(f"{name} must be contiguous along its last dimension")
+    return t.data_ptr()
+
+
+def _f32vec(t: Optional[torch.Tensor], name: str, n: int) -> int:
+    if t is None:
+        return 0
+    if t.numel() != n:
+        raise ValueError(f"{name} must have {n} elements, got {t.numel()}")
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        raise TypeError(f"{name} must be a contiguous fp32 tensor")
+    return _chk(t.reshape(-1), name)
+
+
+def set_variant(op: str, variant: int) -> int:
+    lib = _lib.load()
+    prev = lib.cdm_set_variant(op.encode(), int(variant))
+    if prev < 0:
+        raise RuntimeError(f"set_variant failed: {_lib.last_error()}")
+    return prev
+
+
+# ----------------------------------------------------------------------------- norm / quant
+def adaln_rmsnorm(x: torch.Tensor, w: torch.Tensor, shift: Optional[torch.Tensor] = None,
+                  scale: Optional[torch.Tensor] = None, eps: float = 1e-6,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = rmsnorm(x) * w * (1 + scale) + shift; x [n, d] bf16 contiguous."""
+    lib = _lib.load()
+    n, d = x.shape
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    out = torch.empty_like(x) if out is None else out
+    if not out.is_contiguous() or out.shape != x.shape:
+        raise ValueError("out must be a contiguous tensor of x's shape")
+    rc = lib.cdm_adaln_rmsnorm_bf16(_chk(x, "x", torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
+                                    _f32vec(shift, "shift", d), _f32vec(scale, "scale", d),
+                                    _chk(out, "out", torch.bfloat16, 2), n, d, float(eps), _stream())
+    _lib.check(rc, "cdm_adaln_rmsnorm_bf16")
+    return out
+
+
+def adaln_rmsnorm_quant(x, w, shift=None, scale=None, eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Same norm, output quantised per token to e4m3: returns (yq [n, d] float8_e4m3fn, s_tok [n] fp32)."""
+    lib = _lib.load()
+    n, d = x.shape
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    yq = torch.empty((n, d), dtype=FP8_DTYPE, device=x.device)
+    s = torch.empty((n,), dtype=torch.float32, device=x.device)
+    rc = lib.cdm_adaln_rmsnorm_quant_e4m3(_chk(x, "x", torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
+                                          _f32vec(shift, "shift", d), _f32vec(scale, "scale", d), yq.data_ptr(),
+                                          s.data_ptr(), n, d, float(eps), _stream())
+    _lib.check(rc, "cdm_adaln_rmsnorm_quant_e4m3")
+    return yq, s
+
+
+def quant_rows(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row e4m3 quantisation of a bf16 matrix [rows, cols] (row stride may exceed cols)."""
+    lib = _lib.load()
+    rows, cols = a.shape
+    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=a.device)
+    s = torch.empty((rows,), dtype=torch.float32, device=a.device)
+    rc = lib.cdm_quant_rows_e4m3(_chk(a, "a", torch.bfloat16, 2), a.stride(0), q.data_ptr(), s.data_ptr(), rows, cols,
+                                 _stream())
+    _lib.check(rc, "cdm_quant_rows_e4m3")
+    return q, s
+
+
+# ----------------------------------------------------------------------------- GEMM
+def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, epilogue: str = "none",
+         residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+         cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rope_cols: int = 0,
+         head_dim: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = epilogue(a[M, K] @ w[N, K]^T); bf16 in / fp32 accumulate / bf16 out."""
+    lib = _lib.load()
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or (w2 is not None and w2.shape != w.shape):
+        raise ValueError("weight shape mismatch")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    if out.shape != (M, N):
+        raise ValueError("out shape mismatch")
+    if w2 is not None and w2.stride(0) != w.stride(0):
+        raise ValueError("w and w2 must share a row stride")
+    half = head_dim // 2 if head_dim else 0
+    rc = lib.cdm_gemm_bf16(_chk(a, "a", torch.bfloat16, 2), a.stride(0), _chk(w, "w", torch.bfloat16, 2), w.stride(0),
+                           _chk(w2, "w2", torch.bfloat16, 2), _chk(out, "out", torch.bfloat16, 2), out.stride(0),
+                           M, N, K, _EPI[epilogue], _chk(residual, "residual", torch.bfloat16, 2),
+                           residual.stride(0) if residual is not None else 0, _f32vec(gate, "gate", N),
+                           _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols), int(head_dim),
+                           _stream())
+    _lib.check(rc, "cdm_gemm_bf16")
+    return out
+
+
+def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, *,
+             w2q: Optional[torch.Tensor] = None, sw2: Optional[torch.Tensor] = None, epilogue: str = "none",
+             residual=None, gate=None, cos=None, sin=None, rope_cols: int = 0, head_dim: int = 0,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = epilogue((aq @ wq^T) * sa[:, None] * sw[None, :]); e4m3 operands, bf16 out."""
+    lib = _lib.load()
+    M, K = aq.shape
+    N = wq.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=aq.device)
+    half = head_dim // 2 if head_dim else 0
+    rc = lib.cdm_gemm_fp8(_chk(aq, "aq", FP8_DTYPE, 2), aq.stride(0), _f32vec(sa, "sa", M),
+                          _chk(wq, "wq", FP8_DTYPE, 2), wq.stride(0), _f32vec(sw, "sw", N),
+                          _chk(w2q, "w2q", FP8_DTYPE, 2), _f32vec(sw2, "sw2", N),
+                          _chk(out, "out", torch.bfloat16, 2), out.stride(0), M, N, K, _EPI[epilogue],
+                          _chk(residual, "residual", torch.bfloat16, 2),
+                          residual.stride(0) if residual is not None else 0, _f32vec(gate, "gate", N),
+                          _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols), int(head_dim),
+                          _stream())
+    _lib.check(rc, "cdm_gemm_fp8")
+    return out
+
+
+def grouped_gemm(a: torch.Tensor, ws: Sequence[torch.Tensor], segments: Sequence[Tuple[int, int]], *,
+                 w2s: Optional[Sequence[torch.Tensor]] = None, epilogue: str = "none", residual=None,
+                 gates: Optional[Sequence[Optional[torch.Tensor]]] = None, cos=None, sin=None, rope_cols: int = 0,
+                 head_dim: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """MoT routed linear: rows [start, start+len) of ``a`` use ws[g] (w2s[g], gates[g])."""
+    lib = _lib.load()
+    M, K = a.shape
+    N = ws[0].shape[0]
+    n_seg = len(segments)
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    ldw = ws[0].stride(0)
+    for w in list(ws) + list(w2s or []):
+        if w.shape != ws[0].shape or w.stride(0) != ldw:
+            raise ValueError("all segment weights must share shape and row stride")
+    PP = C.c_void_p * n_seg
+    wp = PP(*[_chk(w, "w", torch.bfloat16, 2) for w in ws])
+    w2p = PP(*[_chk(w, "w2", torch.bfloat16, 2) for w in w2s]) if w2s is not None else None
+    gp = PP(*[(_f32vec(g, "gate", N) or None) for g in gates]) if gates is not None else None
+    I64 = C.c_int64 * n_seg
+    st, ln = I64(*[int(s) for s, _ in segments]), I64(*[int(l) for _, l in segments])
+    half = head_dim // 2 if head_dim else 0
+    rc = lib.cdm_grouped_gemm_bf16(_chk(a, "a", torch.bfloat16, 2), a.stride(0), wp, ldw, w2p,
+                                   _chk(out, "out", torch.bfloat16, 2), out.stride(0), st, ln, n_seg, N, K,
+                                   _EPI[epilogue], _chk(residual, "residual", torch.bfloat16, 2),
+                                   residual.stride(0) if residual is not None else 0, gp,
+                                   _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols),
+                                   int(head_dim), _stream())
+    _lib.check(rc, "cdm_grouped_gemm_bf16")
+    return out
+
+
+# ----------------------------------------------------------------------------- RoPE / attention
+def mrope_qk_(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor, n_heads: int,
+              head_dim: int) -> None:
+    """In-place rotate-half mRoPE on q and k ([n, n_heads*head_dim] views, any row stride)."""
+    lib = _lib.load()
+    n = q.shape[0]
+    half = head_dim // 2
+    rc = lib.cdm_mrope_qk_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _chk(k, "k", torch.bfloat16, 2),
+                               k.stride(0) if k is not None else 0, _f32vec(cos, "cos", n * half),
+                               _f32vec(sin, "sin", n * half), n, n_heads, head_dim, _stream())
+    _lib.check(rc, "cdm_mrope_qk_bf16")
+
+
+def attn_workspace_bytes(n_tokens: int, n_heads: int, head_dim: int) -> int:
+    return int(_lib.load().cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim))
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
+              out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Full non-causal attention; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free)."""
+    lib = _lib.load()
+    n = q.shape[0]
+    d = n_heads * head_dim
+    if q.shape != (n, d) or k.shape != (n, d) or v.shape != (n, d):
+        raise ValueError("q, k, v must be [n_tokens, n_heads*head_dim]")
+    if out is None:
+        out = torch.empty((n, d), dtype=torch.bfloat16, device=q.device)
+    need = attn_workspace_bytes(n, n_heads, head_dim)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    qp, kp, vp = _chk(q, "q", torch.bfloat16, 2), _chk(k, "k", torch.bfloat16, 2), _chk(v, "v", torch.bfloat16, 2)
+    op, wp = _chk(out, "out", torch.bfloat16, 2), _chk(workspace, "workspace", torch.uint8, 1)
+    if _ATTN_TIMER is None:
+        rc = lib.cdm_attn_fwd_bf16(qp, q.stride(0), kp, k.stride(0), vp, v.stride(0), op, out.stride(0), n, n_heads,
+                                   head_dim, wp, workspace.numel(), _stream())
+        _lib.check(rc, "cdm_attn_fwd_bf16")
+        return out
+    # timed form: the same two stages, with HIP events around the attention kernel alone
+    rc = lib.cdm_transpose_v_bf16(vp, v.stride(0), wp, workspace.numel(), n, n_heads, head_dim, _stream())
+    _lib.check(rc, "cdm_transpose_v_bf16")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    rc = lib.cdm_attn_fwd_vt_bf16(qp, q.stride(0), kp, k.stride(0), wp, op, out.stride(0), n, n_heads, head_dim,
+                                  _stream())
+    e1.record()
+    _lib.check(rc, "cdm_attn_fwd_vt_bf16")
+    _ATTN_TIMER.append((e0, e1))
+    return out
+
+
+_ATTN_TIMER = None
+
+
+def time_attention(enable: bool):
+    """Start (True) or stop (False) collecting HIP event pairs around every attention kernel launch on the
+    current stream; stopping returns the list of (start, end) events."""
+    global _ATTN_TIMER
+    prev, _ATTN_TIMER = _ATTN_TIMER, ([] if enable else None)
+    return prev

@@ -1,0 +1,179 @@
+/*
+ * cosmos_dm.h - C ABI of libcosmos_dm_hip.so: hand-written HIP kernels (gfx950 / MI355X)
+ * for the Cosmos 3 Generator-mode diffusion-transformer (DM) block forward.
+ *
+ * The reference repository (NVIDIA/cosmos) has no FFI of its own for this path: it calls
+ * the block through the diffusers pipeline (README.md:238-263,
+ * cookbooks/cosmos3/generator/audiovisual/run_with_diffusers.ipynb:523-612), whose
+ * transformer -> block -> attention-processor forward runs these operators as torch ops
+ * (architecture: README.md:74 and cookbooks/cosmos3/cosmos3-model-architecture.png).
+ * Each entry point below names the operator of that forward it replaces.
+ *
+ * Conventions
+ *   - every function returns 0 (CDM_OK) or a negative cdm_status; cdm_last_error() gives
+ *     a thread-local message for the last failure on the calling thread;
+ *   - all pointers are DEVICE pointers owned by the caller (16-byte aligned unless noted),
+ *     tensors are row-major and bf16 (uint16 storage) unless noted; `ld*` are row strides
+ *     in ELEMENTS;
+ *   - the library never allocates, frees or retains device memory, never synchronises the
+ *     device, and enqueues all work on `stream` (a hipStream_t passed as void*);
+ *   - arguments are validated on the host before any launch.
+ */
+#ifndef COSMOS_DM_H
+#define COSMOS_DM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum cdm_status {
+    CDM_OK = 0,
+    CDM_ERR_BAD_ARG = -1,     /* null pointer, negative size, unknown enum value */
+    CDM_ERR_BAD_SHAPE = -2,   /* size not supported by the kernels (see each function) */
+    CDM_ERR_BAD_ALIGN = -3,   /* pointer or stride not 16-byte aligned */
+    CDM_ERR_NO_DEVICE = -4,   /* no HIP device visible to the process */
+    CDM_ERR_LAUNCH = -5,      /* hipGetLastError() after a launch was not hipSuccess */
+    CDM_ERR_UNSUPPORTED = -6  /* feature combination not built */
+} cdm_status;
+
+/* GEMM epilogues (cdm_gemm_bf16 / cdm_gemm_fp8). */
+typedef enum cdm_epilogue {
+    CDM_EPI_NONE = 0,          /* C = A W^T                                              */
+    CDM_EPI_SWIGLU = 1,        /* C = silu(A Wg^T) * (A Wu^T)          (W = Wg, W2 = Wu) */
+    CDM_EPI_GATE_RESIDUAL = 2, /* C = R + gate[n] * (A W^T)            (gate may be null = 1) */
+    CDM_EPI_ROPE_QK = 3        /* C = A W^T with rotate-half RoPE applied to the columns
+                                  below `rope_cols` (heads of width head_dim)            */
+} cdm_epilogue;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int32_t cdm_version(void);
+
+/* Message for the last non-zero status returned on this thread ("" if none). */
+const char* cdm_last_error(void);
+
+/* Number of HIP devices visible (0 on a host without a GPU); never fails. */
+int32_t cdm_device_count(void);
+
+/*
+ * adaLN-modulated RMSNorm - replaces the per-branch norm + shift/scale modulation at the
+ * head of each half of the block (README.md:74 "per-branch norm"; RMSNorm definition as in
+ * transformers Qwen3VLTextRMSNorm.forward, models/qwen3_vl/modeling_qwen3_vl.py:400-405).
+ *   y[i,j] = x[i,j] * rsqrt(mean_j x[i,:]^2 + eps) * w[j] * (1 + scale[j]) + shift[j]
+ * x, y: [n_tokens, d] bf16 (y may alias x); w: [d] bf16; shift, scale: [d] fp32, either may be
+ * null (plain RMSNorm of the AR branch).  d % 8 == 0, d <= 8192.
+ */
+int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const float* shift, const float* scale,
+                               void* y, int64_t n_tokens, int64_t d, float eps, void* stream);
+
+/*
+ * Same norm with a per-token e4m3 quantisation epilogue (fp8 variant of the block):
+ *   s_tok[i] = max_j |y[i,j]| / 448 (0 -> 1);  yq[i,j] = e4m3(y[i,j] / s_tok[i])
+ * yq: [n_tokens, d] bytes (OCP e4m3fn), s_tok: [n_tokens] fp32.
+ */
+int32_t cdm_adaln_rmsnorm_quant_e4m3(const void* x, const void* w, const float* shift, const float* scale,
+                                     void* yq, float* s_tok, int64_t n_tokens, int64_t d, float eps,
+                                     void* stream);
+
+/*
+ * Per-row dynamic e4m3 quantisation of a bf16 matrix (activations before a quantised linear):
+ *   s[i] = max_j |a[i,j]| / 448 (0 -> 1);  q[i,j] = e4m3(a[i,j] / s[i]).  cols % 8 == 0, cols <= 32768.
+ * Also used offline for weights W[out, in] (per-output-channel scales).
+ */
+int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, float* s, int64_t rows, int64_t cols,
+                            void* stream);
+
+/*
+ * bf16 linear layer(s) with a fused epilogue - replaces nn.Linear (no bias) of the DM branch:
+ * add_q_proj/add_k_proj/add_v_proj (fused as one [3d, d] weight), to_add_out, and the
+ * moe_gen gate/up/down projections (parameter names: transformers
+ * models/cosmos3_omni/modeling_cosmos3_omni.py:39-60).
+ *   A: [M, K] (lda), W: [N, K] (ldw) row-major "out, in" like nn.Linear.weight, C: [M, N] (ldc).
+ *   fp32 accumulation on MFMA, one rounding to bf16 at the end.
+ *   CDM_EPI_SWIGLU:        W = gate_proj.weight, W2 = up_proj.weight (same shape/ld), C: [M, N]
+ *   CDM_EPI_GATE_RESIDUAL: R: [M, N] (ldr) residual (may alias C), gate: [N] fp32 or null
+ *   CDM_EPI_ROPE_QK:       cos, sin: [M, head_dim/2] fp32; columns [0, rope_cols) are rotated
+ *                          per head (pairs (i, i + head_dim/2)); head_dim in {64, 128};
+ *                          rope_cols % 256 == 0
+ * K % 128 == 0; M, N >= 1 arbitrary (N % 8 == 0).
+ */
+int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2,
+                      void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epilogue,
+                      const void* R, int64_t ldr, const float* gate,
+                      const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
+                      void* stream);
+
+/*
+ * fp8 (e4m3) linear with per-token and per-output-channel scales - the quantised variant:
+ *   C[i,j] = sa[i] * sw[j] * sum_k Aq[i,k] Wq[j,k]   (fp32 accumulate) -> bf16, then the epilogue.
+ * Aq: [M, K] bytes, Wq: [N, K] bytes (W2q/sw2 for CDM_EPI_SWIGLU).  K % 256 == 0.
+ */
+int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const void* Wq, int64_t ldw, const float* sw,
+                     const void* W2q, const float* sw2,
+                     void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epilogue,
+                     const void* R, int64_t ldr, const float* gate,
+                     const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
+                     void* stream);
+
+/*
+ * Standalone 3-D mRoPE on Q and K in place - replaces apply_rotary_pos_emb with mRoPE tables
+ * (rotate-half pairs, transformers models/qwen3_vl/modeling_qwen3_vl.py:138-142,412-435;
+ * table layouts :352-388 and models/qwen2_vl/modeling_qwen2_vl.py:212-222).
+ *   q, k: [n_tokens, n_heads, head_dim] with row strides ldq, ldk (elements); k may be null.
+ *   cos, sin: [n_tokens, head_dim/2] fp32 (the axis layout lives entirely in the tables).
+ * head_dim in {64, 128}.
+ */
+int32_t cdm_mrope_qk_bf16(void* q, int64_t ldq, void* k, int64_t ldk, const float* cos, const float* sin,
+                          int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream);
+
+/*
+ * Shared full (non-causal) self-attention over the joint sequence - replaces the attention
+ * processor's scaled_dot_product_attention call (README.md:74; eager form transformers
+ * models/qwen3_vl/modeling_qwen3_vl.py:171-193, fp32 softmax).
+ *   O = softmax(Q K^T / sqrt(head_dim)) V per head, no mask.
+ *   q, k, v: [n_tokens, n_heads, head_dim] with row strides ldq, ldk, ldv; o: [n_tokens, n_heads*head_dim] (ldo).
+ *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds V transposed
+ *   per head); its contents are undefined afterwards.
+ * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
+ */
+int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim);
+int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
+                          void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first
+ * V[n_tokens, n_heads, head_dim] -> vt[n_heads][head_dim][n_tokens rounded up to 64] (zero padded;
+ * vt_bytes >= cdm_attn_workspace_bytes), then the attention kernel proper reading vt.  A caller that
+ * times or profiles the attention kernel alone, or that keeps V transposed across calls, uses these.
+ */
+int32_t cdm_transpose_v_bf16(const void* v, int64_t ldv, void* vt, int64_t vt_bytes, int64_t n_tokens,
+                             int32_t n_heads, int32_t head_dim, void* stream);
+int32_t cdm_attn_fwd_vt_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
+                             void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
+                             void* stream);
+
+/*
+ * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each
+ * (README.md:53,74 - per-modality weights around one shared attention).  Equivalent to
+ * cdm_gemm_bf16 on rows [seg_start[g], seg_start[g] + seg_len[g]) with W[g] (and W2[g], gate[g]).
+ * seg_* are HOST arrays of n_seg entries; W/W2/gate are HOST arrays of n_seg device pointers
+ * (gate[g] may be null = ungated branch).
+ */
+int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw,
+                              const void* const* W2, void* C, int64_t ldc,
+                              const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg,
+                              int64_t N, int64_t K, int32_t epilogue,
+                              const void* R, int64_t ldr, const float* const* gate,
+                              const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
+                              void* stream);
+
+/* Tuning knob for measurements: selects a kernel variant by name ("attn", "gemm"); returns the
+ * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default. */
+int32_t cdm_set_variant(const char* op, int32_t variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COSMOS_DM_H */

@@ -191,9 +191,9 @@ def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> to
     (TF/models/qwen3_vl/modeling_qwen3_vl.py:171-193; non-causal full
     attention for DM tokens per REF/README.md:74).
     """
-    q = q_rows.to(torch.float32).transpose(0, 1)   # [H,R,dh]
-    kk = k.to(torch.float32).transpose(0, 1)       # [H,N,dh]
-    vv = v.to(torch.float32).transpose(0, 1)
+    q = q_rows.to(torch.float32).transpose(0, 1).contiguous()   # [H,R,dh]
+    kk = k.to(torch.float32).transpose(0, 1).contiguous()       # [H,N,dh]
+    vv = v.to(torch.float32).transpose(0, 1).contiguous()
     s = torch.matmul(q, kk.transpose(1, 2)) * (1.0 / math.sqrt(q.shape[-1]))
     p = torch.softmax(s, dim=-1, dtype=torch.float32)
     return torch.matmul(p, vv).transpose(0, 1).contiguous()
@@ -201,8 +201,15 @@ def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> to
 
 def attention(q, k, v, chunk: int = 1024) -> torch.Tensor:
     """Full attention, chunked over query rows so scores are never all resident."""
-    out = [attention_rows(q[i:i + chunk], k, v) for i in range(0, q.shape[0], chunk)]
-    return torch.cat(out, 0)
+    kk = k.to(torch.float32).transpose(0, 1).contiguous()
+    vv = v.to(torch.float32).transpose(0, 1).contiguous()
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    out = []
+    for i in range(0, q.shape[0], chunk):
+        qq = q[i:i + chunk].to(torch.float32).transpose(0, 1).contiguous()
+        p = torch.softmax(torch.matmul(qq, kk.transpose(1, 2)) * scale, dim=-1, dtype=torch.float32)
+        out.append(torch.matmul(p, vv).transpose(0, 1))
+    return torch.cat(out, 0).contiguous()
 
 
 # --------------------------------------------------------------------------

@@ -1,0 +1,75 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares, and
+rejects bad arguments on the host before touching a device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from cosmos_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HAS_GPU = torch.cuda.is_available()
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "cosmos_dm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cdm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = header_functions()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/cosmos_dm.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
+    assert lib.cdm_version() >= 100
+    assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 128 * 2 * 64 * 2
+
+
+def test_bad_arguments_are_rejected_on_the_host():
+    lib = _lib.load()
+    fake = 0x10000   # aligned, never dereferenced: validation fails first
+    assert lib.cdm_adaln_rmsnorm_bf16(None, fake, None, None, fake, 4, 64, 1e-6, None) == _lib.ERR_BAD_ARG
+    assert "null" in _lib.last_error()
+    assert lib.cdm_adaln_rmsnorm_bf16(fake, fake, None, None, fake, 4, 60, 1e-6, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_adaln_rmsnorm_bf16(fake + 2, fake, None, None, fake, 4, 64, 1e-6, None) == _lib.ERR_BAD_ALIGN
+    g = lambda **kw: lib.cdm_gemm_bf16(kw.get("A", fake), kw.get("lda", 128), fake, 128, kw.get("W2", None), fake, 256, 8, 256,
+                                       kw.get("K", 128), kw.get("epi", 0), kw.get("R", None), 256, None, None, None,
+                                       kw.get("rope_cols", 0), kw.get("hd", 0), None)
+    assert g(A=None) == _lib.ERR_BAD_ARG
+    assert g(K=96, lda=96) == _lib.ERR_BAD_SHAPE
+    assert g(epi=7) == _lib.ERR_BAD_ARG
+    assert g(epi=_lib.EPI_SWIGLU) == _lib.ERR_BAD_ARG            # W2 missing
+    assert g(epi=_lib.EPI_GATE_RESIDUAL) == _lib.ERR_BAD_ARG     # R missing
+    assert g(epi=_lib.EPI_ROPE_QK) == _lib.ERR_BAD_ARG           # tables missing
+    assert g(lda=100) == _lib.ERR_BAD_ARG                        # stride < K
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, 64, 16, 1, 48, fake, 1 << 20, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, 64, 16, 1, 64, fake, 16, None) == _lib.ERR_BAD_ARG
+    assert "workspace" in _lib.last_error()
+    assert lib.cdm_mrope_qk_bf16(fake, 64, None, 0, fake, fake, 4, 1, 32, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_quant_rows_e4m3(fake, 128, fake, fake, 4, 100, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_set_variant(b"nope", 0) == _lib.ERR_BAD_ARG
+    # empty inputs are accepted without work
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, 64, 0, 1, 64, None, 0, None) == _lib.OK
+
+
+@pytest.mark.skipif(HAS_GPU, reason="needs a host without a GPU")
+def test_valid_call_without_a_device_reports_no_device():
+    lib = _lib.load()
+    fake = 0x10000
+    assert lib.cdm_device_count() == 0
+    assert lib.cdm_adaln_rmsnorm_bf16(fake, fake, None, None, fake, 4, 64, 1e-6, None) == _lib.ERR_NO_DEVICE
+    assert lib.cdm_gemm_bf16(fake, 128, fake, 128, None, fake, 256, 8, 256, 128, 0, None, 0, None, None, None, 0, 0,
+                             None) == _lib.ERR_NO_DEVICE
+    assert "no HIP device" in _lib.last_error()
+
+
+def test_ops_refuse_cpu_tensors():
+    from cosmos_amd import ops
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.adaln_rmsnorm(x, torch.ones(64, dtype=torch.bfloat16))

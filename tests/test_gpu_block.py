@@ -1,0 +1,189 @@
+"""Block / stack parity with the fp32 CPU oracle: the single-block benchmark configuration (C0), a
+three-branch Mixture-of-Transformers block, a small stack, the fp8 variant, and the full-size
+attention (C1 shape) on sampled query rows."""
+import pytest
+import torch
+
+import oracle as O
+from cosmos_amd import CONFIGS, DMBlock, DMStack, ops, rotary
+from cosmos_amd.config import DMConfig
+from gpu_util import BF16_COS, BF16_REL, FP8_COS, FP8_REL, assert_close, dev, oracle_weights, rand_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def make_block(cfg, seed, randomize_norms=True):
+    blk = DMBlock(cfg.d_model, cfg.n_heads, cfg.head_dim, cfg.hidden, cfg.n_branches, cfg.eps, cfg.fp8, device=dev())
+    g = torch.Generator(device=dev()).manual_seed(seed)
+    blk.reset_parameters(g)
+    if randomize_norms:
+        with torch.no_grad():
+            for p in list(blk.norm1_weight) + list(blk.norm2_weight):
+                p.copy_(1 + 0.2 * torch.randn(p.shape, generator=g, device=dev()))
+            blk.adaLN_modulation.bias.copy_(0.3 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
+    return blk
+
+
+def test_c0_single_block_parity():
+    """Benchmark configuration 0: d=1024, 16x64 heads, hidden 4096, grid 4x16x16, sections 16/24/24."""
+    cfg = CONFIGS["C0"]
+    st = DMStack(cfg, device=dev())
+    st.reset_parameters()
+    g = torch.Generator().manual_seed(cfg.seed)
+    x, xr = rand_bf16((cfg.n_tokens, cfg.d_model), g)
+    t = torch.rand(1, generator=g) * 1000.0
+    (y,) = st(x.unsqueeze(0), t.to(dev()))
+    # oracle: same weights in fp32, conditioning through the oracle's own embedding / MLP
+    te = st.time_embedder
+    c = O.time_mlp(O.timestep_embedding(t), te.linear_1.weight.float().cpu(), te.linear_1.bias.float().cpu(),
+                   te.linear_2.weight.float().cpu(), te.linear_2.bias.float().cpu())
+    blk = st.blocks[0]
+    mod = O.adaln_modulation(c, blk.adaLN_modulation.weight.float().cpu(), blk.adaLN_modulation.bias.float().cpu())
+    pos = O.vision_positions(0, cfg.grid)
+    cos, sin = O.mrope_cos_sin(pos, cfg.head_dim, cfg.mrope_sections, cfg.rope_base, cfg.rope_layout)
+    want = O.dm_block(xr, oracle_weights(blk, 1), mod, cos, sin, cfg.n_heads)
+    assert_close(y[0], want, BF16_COS, BF16_REL, "C0 block")
+    # With N(0, 0.02) weights and zero biases the adaLN gates are nearly zero and the block is close to the
+    # identity, so repeat with order-one modulation (gates included) and check the UPDATE y - x as well.
+    gm = torch.Generator().manual_seed(99)
+    strong = [torch.randn(cfg.d_model, generator=gm) * s for s in (0.5, 0.5, 8.0, 0.5, 0.5, 8.0)]
+    y2 = blk(x, None, st.rotary(dev()), modulation=[m.to(dev()) for m in strong])
+    want2 = O.dm_block(xr, oracle_weights(blk, 1), strong, cos, sin, cfg.n_heads)
+    assert float((want2 - xr).abs().max()) > 1.0
+    assert_close(y2, want2, BF16_COS, BF16_REL, "C0 block, strong modulation")
+    assert_close(y2.float().cpu() - xr, want2 - xr, 0.999, BF16_REL, "C0 block update")
+
+
+def test_block_gate_zero_is_identity():
+    cfg = DMConfig("t", 256, 2, 128, 512, 1, (2, 4, 8))
+    blk = make_block(cfg, 3)
+    g = torch.Generator().manual_seed(3)
+    x, _ = rand_bf16((cfg.n_tokens, 256), g)
+    pos, _ = rotary.build_positions(0, cfg.grid)
+    rot = rotary.rotary_tables(pos, 128, cfg.mrope_sections, device=dev())
+    z, o = torch.zeros(256, device=dev()), torch.ones(256, device=dev())
+    y = blk(x, None, rot, modulation=(o, o, z, o, o, z))
+    assert torch.equal(y, x)
+
+
+def test_mot_three_branch_block():
+    cfg = DMConfig("mot", 256, 2, 128, 512, 1, (2, 4, 8), n_text=40, n_action=24, n_branches=3)
+    st = DMStack(cfg, device=dev())
+    blk = make_block(cfg, 11)
+    g = torch.Generator().manual_seed(11)
+    x, xr = rand_bf16((cfg.n_tokens, 256), g)
+    temb, tembr = rand_bf16((256,), g)
+    rot = st.rotary(dev())
+    segs = st.segments()
+    assert segs == [(0, 40, 0, False), (40, 64, 1, True), (104, 24, 2, True)]
+    y = blk(x, temb, rot, segs)
+    mod = O.adaln_modulation(tembr.view(1, -1), blk.adaLN_modulation.weight.float().cpu(),
+                             blk.adaLN_modulation.bias.float().cpu())
+    pos = O.joint_positions([("text", 40), ("video", cfg.grid), ("action", 24)])
+    cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+    ws = oracle_weights(blk, 3)
+    want = O.dm_block(xr, ws, mod, cos, sin, 2, segs)
+    assert_close(y, want, BF16_COS, BF16_REL, "MoT block")
+    # equal weight sets, everything modulated == single-branch block on the same kernels
+    with torch.no_grad():
+        for plist in (blk.attn.qkv_weight, blk.attn.out_weight, blk.norm1_weight, blk.norm2_weight, blk.gate_weight,
+                      blk.up_weight, blk.down_weight):
+            for b in (0, 2):
+                plist[b].copy_(plist[1])
+    y3 = blk(x, temb, rot, [(0, 40, 0, True), (40, 64, 1, True), (104, 24, 2, True)])
+    y1 = blk(x, temb, rot, [(0, cfg.n_tokens, 1, True)])
+    assert_close(y3, y1.float().cpu(), 0.99999, 2e-3, "equal weights == single branch")
+
+
+def test_small_stack_and_encoder_path():
+    cfg = DMConfig("s", 256, 4, 64, 640, 3, (2, 3, 10), n_text=20, mrope_sections=(16, 24, 24))
+    st = DMStack(cfg, device=dev())
+    st.reset_parameters(5)
+    g = torch.Generator().manual_seed(5)
+    xv, xvr = rand_bf16((1, cfg.n_video, 256), g)
+    xt, xtr = rand_bf16((1, cfg.n_text, 256), g)
+    t = torch.tensor([417.0])
+    out = st(xv, t.to(dev()), encoder_hidden_states=xt, return_dict=True)
+    te = st.time_embedder
+    c = O.time_mlp(O.timestep_embedding(t), te.linear_1.weight.float().cpu(), te.linear_1.bias.float().cpu(),
+                   te.linear_2.weight.float().cpu(), te.linear_2.bias.float().cpu())
+    mods = [O.adaln_modulation(c, b.adaLN_modulation.weight.float().cpu(), b.adaLN_modulation.bias.float().cpu())
+            for b in st.blocks]
+    pos = O.joint_positions([("text", cfg.n_text), ("video", cfg.grid)])
+    cos, sin = O.mrope_cos_sin(pos, 64, cfg.mrope_sections)
+    want = O.dm_stack(torch.cat([xtr[0], xvr[0]]), [oracle_weights(b, 1) for b in st.blocks], mods, cos, sin, 4,
+                      st.segments())
+    assert_close(out["joint"], want, BF16_COS, BF16_REL, "3-block stack (joint)")
+    assert_close(out["sample"][0], want[cfg.n_text:], BF16_COS, BF16_REL, "3-block stack (video part)")
+
+
+def test_attention_processor_diffusers_call_shape():
+    """processor(attn, hidden_states, encoder_hidden_states=..., image_rotary_emb=...) -> (hidden, encoder)."""
+    cfg = DMConfig("p", 256, 2, 128, 512, 1, (1, 4, 8), n_text=16, n_branches=2)
+    blk = make_block(cfg, 21, randomize_norms=False)
+    g = torch.Generator().manual_seed(21)
+    h, hr = rand_bf16((1, 32, 256), g)
+    e, er = rand_bf16((1, 16, 256), g)
+    pos, _ = rotary.build_positions(16, cfg.grid)
+    cos, sin = rotary.rotary_tables(pos, 128, cfg.mrope_sections)
+    ho, eo = blk.attn(h, encoder_hidden_states=e, image_rotary_emb=(cos.to(dev()), sin.to(dev())))
+    assert ho.shape == (1, 32, 256) and eo.shape == (1, 16, 256)
+    ws = oracle_weights(blk, 2)
+    xr = torch.cat([er[0], hr[0]])
+    q = torch.cat([xr[:16] @ ws[0]["wq"].t(), xr[16:] @ ws[1]["wq"].t()]); k = torch.cat([xr[:16] @ ws[0]["wk"].t(), xr[16:] @ ws[1]["wk"].t()])
+    v = torch.cat([xr[:16] @ ws[0]["wv"].t(), xr[16:] @ ws[1]["wv"].t()])
+    o = O.attention(O.apply_mrope(q.view(48, 2, 128), cos, sin), O.apply_mrope(k.view(48, 2, 128), cos, sin), v.view(48, 2, 128)).reshape(48, 256)
+    assert_close(eo[0], o[:16] @ ws[0]["wo"].t(), BF16_COS, BF16_REL, "processor encoder stream")
+    assert_close(ho[0], o[16:] @ ws[1]["wo"].t(), BF16_COS, BF16_REL, "processor hidden stream")
+    with pytest.raises(NotImplementedError):
+        blk.attn(h, attention_mask=torch.ones(1, 32, device=dev()), image_rotary_emb=(cos.to(dev()), sin.to(dev())))
+
+
+def test_fp8_block_vs_fp32_oracle():
+    cfg = DMConfig("f8", 512, 4, 128, 1024, 1, (2, 8, 16), n_text=32, fp8=True)
+    st = DMStack(cfg, device=dev())
+    blk = make_block(cfg, 17)
+    g = torch.Generator().manual_seed(17)
+    x, xr = rand_bf16((cfg.n_tokens, 512), g)
+    temb, tembr = rand_bf16((512,), g)
+    y = blk(x, temb, st.rotary(dev()), st.segments())
+    mod = O.adaln_modulation(tembr.view(1, -1), blk.adaLN_modulation.weight.float().cpu(),
+                             blk.adaLN_modulation.bias.float().cpu())
+    pos = O.joint_positions([("text", 32), ("video", cfg.grid)])
+    cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+    ws = oracle_weights(blk, 1)
+    want32 = O.dm_block(xr, ws, mod, cos, sin, 4, st.segments())
+    assert_close(y, want32, FP8_COS, FP8_REL, "fp8 block vs fp32 unquantised oracle")
+    want8 = O.dm_block(xr, ws, mod, cos, sin, 4, st.segments(), fp8=True)
+    assert_close(y, want8, 0.9995, 3e-2, "fp8 block vs quantised oracle")
+
+
+def test_c1_full_size_attention_sampled_rows():
+    """Benchmark configuration 1: 32 heads x 128, grid 16x44x80 = 56,320 tokens, mRoPE 32/48/48, bf16.
+    Attention rows are independent given K and V, so exact fp32 attention on sampled query rows is an exact
+    check of those rows."""
+    cfg = CONFIGS["C1"]
+    n, H, hd, d = cfg.n_tokens, cfg.n_heads, cfg.head_dim, cfg.d_model
+    g = torch.Generator(device=dev()).manual_seed(cfg.seed)
+    qkv = (torch.randn((n, 3 * d), generator=g, device=dev()) / (hd ** 0.5)).to(torch.bfloat16)
+    pos, _ = rotary.build_positions(0, cfg.grid)
+    cos, sin = rotary.rotary_tables(pos, hd, cfg.mrope_sections)
+    pre = qkv.clone()
+    q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
+    ops.mrope_qk_(q, k, cos.to(dev()), sin.to(dev()), H, hd)
+    o = ops.attention(q, k, v, H, hd)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.tensor([0, 1, 31, 32, 255, 256, n - 1, n - 64]),
+                      torch.randint(0, n, (56,), generator=torch.Generator().manual_seed(1))])
+    heads = [0, 13, 31]                                       # three heads keep the CPU side to a few seconds
+    for h in heads:
+        sl = slice(h * hd, (h + 1) * hd)
+        kr = O.apply_mrope(pre[:, d + h * hd:d + (h + 1) * hd].float().cpu().view(n, 1, hd), cos, sin)
+        qr = O.apply_mrope(pre[rows.to(dev()), sl].float().cpu().view(-1, 1, hd), cos[rows], sin[rows])
+        vr = pre[:, 2 * d + h * hd:2 * d + (h + 1) * hd].float().cpu().view(n, 1, hd)
+        want = O.attention_rows(qr, kr, vr).reshape(-1, hd)
+        assert_close(o[rows.to(dev()), sl], want, BF16_COS, BF16_REL, f"C1 attention head {h}")
+    # size-independent property on the whole output: every output row is a convex combination of V rows
+    vmin, vmax = v.float().amin(0), v.float().amax(0)
+    of = o.float()
+    assert bool((of >= vmin - 1e-2).all()) and bool((of <= vmax + 1e-2).all())

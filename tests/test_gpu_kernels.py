@@ -1,0 +1,236 @@
+"""Parity of each HIP kernel (through the C ABI) with the fp32 CPU oracle on identical seeded inputs.
+Tolerances: cos >= 0.999 and max|a-b|/max|b| <= 2e-2 for bf16, <= 5e-2 for fp8 (most checks are much tighter)."""
+import math
+
+import pytest
+import torch
+
+import oracle as O
+from cosmos_amd import ops, rotary
+from gpu_util import assert_close, dev, rand_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------ adaLN RMSNorm
+@pytest.mark.parametrize("n,d", [(1, 64), (37, 1024), (300, 4096), (5, 8192), (9, 1160)])
+@pytest.mark.parametrize("modulated", [True, False])
+def test_adaln_rmsnorm(n, d, modulated):
+    g = gen(n * 7 + d)
+    x, xr = rand_bf16((n, d), g, 2.0)
+    w, wr = rand_bf16((d,), g)
+    sh = torch.randn(d, generator=g) if modulated else None
+    sc = torch.randn(d, generator=g) * 0.5 if modulated else None
+    y = ops.adaln_rmsnorm(x, w, sh.to(dev()) if modulated else None, sc.to(dev()) if modulated else None, 1e-6)
+    want = O.adaln_rms_norm(xr, wr, sh, sc, 1e-6)
+    assert_close(y, want, 0.99999, 6e-3, f"adaln_rmsnorm {n}x{d}")
+    # in place (y aliases x) gives the same bits
+    y2 = ops.adaln_rmsnorm(x, w, sh.to(dev()) if modulated else None, sc.to(dev()) if modulated else None, 1e-6, out=x)
+    assert torch.equal(y2, y)
+
+
+def test_adaln_rmsnorm_closed_form():
+    d = 512
+    x = torch.full((3, d), 2.5, dtype=torch.bfloat16, device=dev())
+    w = torch.linspace(0.5, 1.5, d).to(torch.bfloat16)
+    sc, sh = torch.linspace(-0.2, 0.3, d), torch.linspace(-1, 1, d)
+    y = ops.adaln_rmsnorm(x, w.to(dev()), sh.to(dev()), sc.to(dev()), 0.0)
+    want = (w.float() * (1 + sc) + sh).expand(3, d)
+    assert_close(y, want, 0.99999, 5e-3, "constant rows")
+
+
+# ------------------------------------------------------------------ mRoPE
+@pytest.mark.parametrize("hd,H,sections", [(64, 16, (16, 24, 24)), (128, 4, (32, 48, 48))])
+def test_mrope_standalone(hd, H, sections):
+    g = gen(hd)
+    pos, _ = rotary.build_positions(5, (3, 4, 6), 2)
+    n = pos.shape[1]
+    cos, sin = rotary.rotary_tables(pos, hd, sections)
+    qkv, qkvr = rand_bf16((n, 3 * H * hd), g)
+    d = H * hd
+    q, k = qkv[:, :d], qkv[:, d:2 * d]
+    ops.mrope_qk_(q, k, cos.to(dev()), sin.to(dev()), H, hd)
+    want_q = O.apply_mrope(qkvr[:, :d].view(n, H, hd), cos, sin).reshape(n, d)
+    want_k = O.apply_mrope(qkvr[:, d:2 * d].view(n, H, hd), cos, sin).reshape(n, d)
+    assert_close(qkv[:, :d], want_q, 0.99999, 6e-3, "rope q")
+    assert_close(qkv[:, d:2 * d], want_k, 0.99999, 6e-3, "rope k")
+    assert torch.equal(qkv[:, 2 * d:].float().cpu(), qkvr[:, 2 * d:])      # V untouched
+    # position 0 everywhere is the identity
+    z = torch.zeros(n, hd // 2, device=dev())
+    before = qkv.clone()
+    ops.mrope_qk_(q, None, z.cos(), z.sin(), H, hd)
+    assert torch.equal(before, qkv)
+
+
+# ------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (8, 8, 128), (300, 264, 256), (1024, 3072, 1024), (515, 1000, 384)])
+def test_gemm_plain(M, N, K):
+    g = gen(M + N + K)
+    a, ar = rand_bf16((M, K), g)
+    w, wr = rand_bf16((N, K), g, 0.05)
+    c = ops.gemm(a, w)
+    assert_close(c, ar @ wr.t(), 0.99999, 6e-3, f"gemm {M}x{N}x{K}")
+
+
+def test_gemm_strided_views_and_determinism():
+    g = gen(5)
+    big, bigr = rand_bf16((200, 640), g)
+    w, wr = rand_bf16((520, 256), g, 0.05)
+    a = big[:, 128:384]                                   # row stride 640, K = 256
+    out = torch.zeros((200, 1040), dtype=torch.bfloat16, device=dev())
+    ops.gemm(a, w, out=out[:, 520:])
+    assert_close(out[:, 520:], bigr[:, 128:384] @ wr.t(), 0.99999, 6e-3, "strided gemm")
+    assert float(out[:, :520].abs().max()) == 0.0
+    c1, c2 = ops.gemm(a, w), ops.gemm(a, w)
+    assert torch.equal(c1, c2)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 128, 128), (333, 200, 256), (1024, 4096, 1024)])
+def test_gemm_swiglu(M, N, K):
+    g = gen(M * 3 + N)
+    a, ar = rand_bf16((M, K), g)
+    wg, wgr = rand_bf16((N, K), g, 0.05)
+    wu, wur = rand_bf16((N, K), g, 0.05)
+    c = ops.gemm(a, wg, w2=wu, epilogue="swiglu")
+    want = torch.nn.functional.silu(ar @ wgr.t()) * (ar @ wur.t())
+    assert_close(c, want, 0.99999, 6e-3, f"swiglu {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K,gated", [(256, 256, 128, True), (300, 1024, 512, True), (77, 264, 128, False)])
+def test_gemm_gate_residual(M, N, K, gated):
+    g = gen(M + 11 * N)
+    a, ar = rand_bf16((M, K), g)
+    w, wr = rand_bf16((N, K), g, 0.05)
+    r, rr = rand_bf16((M, N), g)
+    gate = torch.randn(N, generator=g) if gated else None
+    want = rr + (gate if gated else 1.0) * (ar @ wr.t())
+    c = ops.gemm(a, w, epilogue="gate_residual", residual=r, gate=gate.to(dev()) if gated else None)
+    assert_close(c, want, 0.99999, 6e-3, "gate_residual")
+    # in place on the residual stream
+    ops.gemm(a, w, epilogue="gate_residual", residual=r, gate=gate.to(dev()) if gated else None, out=r)
+    assert torch.equal(r, c)
+
+
+@pytest.mark.parametrize("hd,H,sections", [(64, 4, (16, 24, 24)), (128, 2, (32, 48, 48))])
+def test_gemm_rope_qk(hd, H, sections):
+    g = gen(hd + H)
+    d = H * hd                                           # 256
+    pos, _ = rotary.build_positions(7, (3, 5, 8), 3)     # 130 tokens: ragged M
+    n = pos.shape[1]
+    cos, sin = rotary.rotary_tables(pos, hd, sections)
+    a, ar = rand_bf16((n, 128), g)
+    w, wr = rand_bf16((3 * d, 128), g, 0.1)
+    c = ops.gemm(a, w, epilogue="rope_qk", cos=cos.to(dev()), sin=sin.to(dev()), rope_cols=2 * d, head_dim=hd)
+    lin = ar @ wr.t()
+    want = torch.cat([O.apply_mrope(lin[:, :d].view(n, H, hd), cos, sin).reshape(n, d),
+                      O.apply_mrope(lin[:, d:2 * d].view(n, H, hd), cos, sin).reshape(n, d), lin[:, 2 * d:]], 1)
+    assert_close(c[:, :2 * d], want[:, :2 * d], 0.99999, 6e-3, "rope_qk q,k")
+    assert_close(c[:, 2 * d:], want[:, 2 * d:], 0.99999, 6e-3, "rope_qk v")
+
+
+def test_grouped_gemm_three_segments():
+    g = gen(77)
+    K, N = 256, 264
+    segs = [(0, 40), (40, 300), (340, 24)]
+    a, ar = rand_bf16((364, K), g)
+    ws = [rand_bf16((N, K), g, 0.05) for _ in range(3)]
+    r, rr = rand_bf16((364, N), g)
+    gates = [None, torch.randn(N, generator=g), torch.randn(N, generator=g)]
+    c = ops.grouped_gemm(a, [w[0] for w in ws], segs, epilogue="gate_residual", residual=r,
+                         gates=[None if x is None else x.to(dev()) for x in gates])
+    want = torch.cat([rr[s:s + l] + (1.0 if gates[i] is None else gates[i]) * (ar[s:s + l] @ ws[i][1].t())
+                      for i, (s, l) in enumerate(segs)])
+    assert_close(c, want, 0.99999, 6e-3, "grouped gemm")
+
+
+# ------------------------------------------------------------------ attention
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n,H,hd", [(64, 2, 64), (256, 1, 128), (1000, 3, 128), (321, 2, 64), (1, 1, 128), (130, 2, 128)])
+def test_attention_vs_oracle(n, H, hd, variant):
+    g = gen(n + H + hd)
+    d = H * hd
+    qkv, qkvr = rand_bf16((n, 3 * d), g, 1.5)
+    prev = ops.set_variant("attn", variant)
+    try:
+        o = ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], H, hd)
+    finally:
+        ops.set_variant("attn", prev)
+    want = O.attention(qkvr[:, :d].view(n, H, hd), qkvr[:, d:2 * d].view(n, H, hd), qkvr[:, 2 * d:].view(n, H, hd))
+    assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"attention n={n} H={H} hd={hd} variant={variant}")
+
+
+def test_attention_closed_forms_and_determinism():
+    g = gen(9)
+    n, H, hd = 200, 2, 128
+    d = H * hd
+    q, _ = rand_bf16((n, d), g)
+    k, _ = rand_bf16((n, d), g)
+    v, vr = rand_bf16((1, d), g)
+    vc = v.expand(n, d).contiguous()
+    o = ops.attention(q, k, vc, H, hd)                    # V constant over keys -> output equals it
+    assert_close(o, vr.expand(n, d), 0.99999, 5e-3, "V const")
+    v2, v2r = rand_bf16((n, d), g)
+    o1 = ops.attention(torch.zeros_like(q), k, v2, H, hd)  # zero queries -> mean of V
+    assert_close(o1, v2r.mean(0, keepdim=True).expand(n, d), 0.9999, 1e-2, "uniform softmax")
+    perm = torch.randperm(n, generator=g).to(dev())
+    a, b = ops.attention(q, k, v2, H, hd), ops.attention(q, k[perm].contiguous(), v2[perm].contiguous(), H, hd)
+    assert_close(a, b.float().cpu(), 0.9999, 1e-2, "key permutation")
+    assert torch.equal(a, ops.attention(q, k, v2, H, hd))
+
+
+# ------------------------------------------------------------------ fp8
+@pytest.mark.parametrize("rows,cols", [(5, 64), (300, 4096), (17, 1160)])
+def test_quant_rows_exact(rows, cols):
+    g = gen(rows + cols)
+    a, ar = rand_bf16((rows, cols), g, 3.0)
+    a[0].zero_(); ar[0].zero_()
+    q, s = ops.quant_rows(a)
+    wq, ws = O.quant_e4m3_rows(ar)
+    assert torch.equal(s.cpu(), ws.reshape(-1))
+    assert torch.equal(q.float().cpu(), wq)
+
+
+def test_adaln_rmsnorm_quant():
+    g = gen(31)
+    n, d = 70, 1024
+    x, xr = rand_bf16((n, d), g, 2.0)
+    w, wr = rand_bf16((d,), g)
+    sh, sc = torch.randn(d, generator=g), torch.randn(d, generator=g) * 0.5
+    yq, s = ops.adaln_rmsnorm_quant(x, w, sh.to(dev()), sc.to(dev()), 1e-6)
+    want = O.adaln_rms_norm(xr, wr, sh, sc, 1e-6)
+    assert_close(yq.float() * s[:, None], want, 0.999, 5e-2, "norm+quant dequantised")
+    # consistent with the two-kernel route (norm to bf16, then quantise)
+    y = ops.adaln_rmsnorm(x, w, sh.to(dev()), sc.to(dev()), 1e-6)
+    q2, s2 = ops.quant_rows(y)
+    assert torch.equal(s, s2) and torch.equal(yq.float(), q2.float())
+
+
+@pytest.mark.parametrize("M,N,K,epi", [(256, 256, 256, "none"), (300, 520, 512, "none"), (300, 264, 256, "swiglu"),
+                                       (130, 256, 256, "gate_residual")])
+def test_gemm_fp8(M, N, K, epi):
+    g = gen(M + N + K + len(epi))
+    a, ar = rand_bf16((M, K), g)
+    w, wr = rand_bf16((N, K), g, 0.05)
+    aq, sa = ops.quant_rows(a)
+    wq, sw = ops.quant_rows(w)
+    lin = lambda A, W: O.fp8_linear(A, W)
+    if epi == "none":
+        c = ops.gemm_fp8(aq, sa, wq, sw)
+        want, ref32 = lin(ar, wr), ar @ wr.t()
+    elif epi == "swiglu":
+        w2, w2r = rand_bf16((N, K), g, 0.05)
+        w2q, sw2 = ops.quant_rows(w2)
+        c = ops.gemm_fp8(aq, sa, wq, sw, w2q=w2q, sw2=sw2, epilogue="swiglu")
+        want = torch.nn.functional.silu(lin(ar, wr)) * lin(ar, w2r)
+        ref32 = torch.nn.functional.silu(ar @ wr.t()) * (ar @ w2r.t())
+    else:
+        r, rr = rand_bf16((M, N), g)
+        gate = torch.randn(N, generator=g)
+        c = ops.gemm_fp8(aq, sa, wq, sw, epilogue="gate_residual", residual=r, gate=gate.to(dev()))
+        want, ref32 = rr + gate * lin(ar, wr), rr + gate * (ar @ wr.t())
+    assert_close(c, want, 0.99999, 6e-3, f"fp8 gemm vs quantised oracle ({epi})")
+    assert_close(c, ref32, 0.999, 5e-2, f"fp8 gemm vs fp32 ({epi})")
