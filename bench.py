@@ -66,6 +66,7 @@ def main():
     ap.add_argument("--workload", default="C2", choices=["C0", "C2", "C3", "C4"])
     ap.add_argument("--blocks", type=int, default=0, help="override the number of blocks (measurement aid; 0 = config)")
     ap.add_argument("--attn-variant", type=int, default=0)
+    ap.add_argument("--gemm-variant", type=int, default=0)
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -86,6 +87,7 @@ def main():
         cfg = dataclasses.replace(cfg, n_blocks=args.blocks)
     _lib.load()
     ops.set_variant("attn", args.attn_variant)
+    ops.set_variant("gemm", args.gemm_variant)
 
     stack = DMStack(cfg, device=dev)
     stack.reset_parameters()
@@ -112,6 +114,8 @@ def main():
 
     ms_per_step = wall * 1e3 / args.steps
     attn_ms = [a.elapsed_time(b) for a, b in events]
+    if not attn_ms:      # measurement variants of the attention kernel are timed as a whole by rocprof only
+        attn_ms = [float("nan")]
     attn_avg_ms = sum(attn_ms) / len(attn_ms)
     attn_flops = cfg.attn_flops_per_block()
     attn_tflops = attn_flops / (attn_avg_ms * 1e-3) / 1e12
@@ -126,7 +130,7 @@ def main():
         "config": {"workload": f"{cfg.name}: {cfg.n_blocks} DM blocks, d={cfg.d_model}, {cfg.n_heads}x{cfg.head_dim} heads, "
                                f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
-                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant},
+                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4), "traffic": None,
                      "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},

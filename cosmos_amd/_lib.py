@@ -36,8 +36,8 @@ SIGNATURES = {
     "cdm_mrope_qk_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I32, _I32, _P]),
     "cdm_attn_workspace_bytes": (_I64, [_I64, _I32, _I32]),
     "cdm_attn_fwd_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I32, _I32, _P, _I64, _P]),
-    "cdm_transpose_v_bf16": (_I32, [_P, _I64, _P, _I64, _I64, _I32, _I32, _P]),
-    "cdm_attn_fwd_vt_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _I32, _I32, _P]),
+    "cdm_attn_pack_kv_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _I64, _I32, _I32, _P]),
+    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _I64, _I64, _I32, _I32, _P]),
     "cdm_grouped_gemm_bf16": (_I32, [_P, _I64, C.POINTER(_P), _I64, C.POINTER(_P), _P, _I64, C.POINTER(_I64),
                                      C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P, _P, _I64,
                                      _I32, _P]),
@@ -45,7 +45,8 @@ SIGNATURES = {
 
 
 def lib_path() -> str:
-    return _build.LIB_PATH
+    """Path of the shared library; COSMOS_DM_LIB overrides the in-tree build (e.g. an experimental build)."""
+    return os.environ.get("COSMOS_DM_LIB") or _build.LIB_PATH
 
 
 def load():

@@ -275,6 +275,329 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Software-pipelined kernel (8 waves x 32 query rows) over PRE-TILED K and V.
+//  * K and V are first re-laid out in the workspace as the exact LDS image of each 64-key tile,
+//    chunk-major:  Kp[head][tile][c = dh/8][key r = 0..63][8 ch]   and
+//                  Vp[head][tile][c = key/8 (0..7)][channel row = 0..HD-1][8 keys]  (V transposed).
+//    A tile is then one contiguous 16 KB (HD=128) stream for the direct-to-LDS loads, every fragment
+//    read is  lane_base + compile-time offset  (no swizzle arithmetic, two address registers in
+//    total) and 16 consecutive lanes always read 16 distinct 16-byte slots (no bank conflicts).
+//    Keys beyond n_tokens are zero in the workspace and masked to -inf in the last tile.
+//  * the scores of tile j+1 (S^T = K Q^T, 16 MFMAs) are issued BEFORE the softmax of tile j, so one
+//    wave always has matrix work in flight under its own exp/convert VALU work;
+//  * Q is pre-multiplied by log2(e)/sqrt(dh) and the score accumulators start at -m_ref instead of 0,
+//    so a score leaves the MFMA already shifted and p = exp2(S) needs no per-score FMA;
+//  * m_ref is a running reference that only moves when a row's tile maximum exceeds it by more than
+//    2^kGrowLog2 (then O and l are rescaled: exact, merely a different reference);
+//  * the row sum uses v_dot2c_f32_bf16 on the packed probabilities (2 values per instruction).
+// ---------------------------------------------------------------------------------------------
+constexpr float kGrowLog2 = 4.0f;
+
+// Q fragments 0..QREG-1 stay in registers; the others are parked in a per-lane LDS slot (each lane re-reads
+// exactly the 16 bytes it wrote, so no barrier is involved) to keep the kernel inside 256 registers.
+template <int HD>
+struct QSplit {
+    static constexpr int KS = HD / 16;
+    static constexpr int QREG = KS;     // all of Q fits since the step exists in a single copy
+    static constexpr int QLDS = KS - QREG;
+};
+
+template <int HD>
+__device__ __forceinline__ void scores_tile(const char* sk, const bf16x8 (&qf)[QSplit<HD>::QREG], const char* qstash,
+                                            f32x16 (&s)[2], int lane) {
+    // s holds the accumulator start values (-reference, or -inf for keys beyond the sequence end)
+    constexpr int QREG = QSplit<HD>::QREG;
+    // lane reads key row pi(lane%32) (+32 for the second block), chunk 2ks + lane/32
+    const char* base = sk + (lane >> 5) * 1024 + key_perm(lane & 31) * 16;
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks) {
+        bf16x8 q;
+        if (ks < QREG) q = qf[ks];
+        else q = *reinterpret_cast<const bf16x8*>(qstash + (ks - QREG) * 1024);
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + ks * 2048 + kvb * 512);
+            s[kvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q, s[kvb], 0, 0, 0);
+        }
+    }
+}
+
+// Accumulator start values of a score tile: `start` everywhere, or -inf for keys >= keys_valid (ragged last
+// tile).  Register v of block kvb holds key 32 kvb + 16 (v/8) + 8 (lane/32) + v%8: the compile-time part is
+// compared against ONE per-lane threshold so that no per-register key index is ever materialised.
+__device__ __forceinline__ void init_scores(f32x16 (&s)[2], float start, bool ragged, int keys_valid, int lane) {
+    if (ragged) {      // wave-uniform
+        const int thr = keys_valid - 8 * (lane >> 5);
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int kc = 32 * kvb + 16 * (v >> 3) + (v & 7);
+                s[kvb][v] = (kc >= thr) ? -INFINITY : start;
+            }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { s[0][v] = start; s[1][v] = start; }
+    }
+}
+
+__device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
+    float mx = __builtin_fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = __builtin_fmaxf(__builtin_fmaxf(mx, s[0][v]), s[1][v]);   // v_max3_f32
+    return __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
+}
+
+// One pipeline step.  s_cur (scores of tile j, accumulated on top of -m_ref) and mx_cur (its row maximum,
+// already reduced over the wave halves) come from the previous step.
+//   top      : rare branch - if a row maximum exceeds the reference by more than 2^kGrowLog2, move the reference
+//   block A  : S(j+1) MFMAs  ||  exp2 / bf16 pack / row-sum of tile j           (VALU under MFMA)
+//   block B  : O^T += V^T P^T MFMAs  ||  row maximum of S(j+1) for the next step
+template <int HD>
+__device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cur,
+                                          const bf16x8 (&qf)[QSplit<HD>::QREG], const char* qstash,
+                                          f32x16 (&s_cur)[2], f32x16 (&s_next)[2], f32x16 (&oacc)[HD / 32],
+                                          float& m_ref, float& mx_cur, float& l_run, int lane, bool next_ragged,
+                                          int next_keys_valid) {
+    if (__builtin_amdgcn_ballot_w64(mx_cur > kGrowLog2) != 0) {
+        const float delta = mx_cur > kGrowLog2 ? mx_cur : 0.0f;
+        const float fac = __builtin_amdgcn_exp2f(-delta);
+        m_ref += delta;
+        l_run *= fac;
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_cur[kvb][v] -= delta;
+#pragma unroll
+        for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[t][v] *= fac;
+    }
+    init_scores(s_next, -m_ref, next_ragged, next_keys_valid, lane);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K buffer and
+    // their result is never used - cheaper than a second copy of the step.)
+    scores_tile<HD>(sk_next, qf, qstash, s_next, lane);
+    bf16x8 pf[4];
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    float psum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        bf16x8 p8;
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            bf16x2 pp;
+            pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e]);
+            pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e + 1]);
+            psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
+            p8[e] = pp[0];
+            p8[e + 1] = pp[1];
+        }
+        pf[j] = p8;
+    }
+    l_run += psum;
+    // 16 MFMAs, 16 + QLDS fragment reads, ~64 VALU: a few reads up front, then per MFMA one or two reads and
+    // four VALU instructions
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < QSplit<HD>::QLDS; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+#pragma unroll
+    for (int i = QSplit<HD>::QLDS; i < 2 * (HD / 16); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- block B: lane reads channel row 32t + lane%32, key chunk 2j + lane/32
+    const char* vb = sv_cur + (lane >> 5) * (HD * 16) + (lane & 31) * 16;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < HD / 32; ++t) {
+            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vb + j * (HD * 32) + t * 512);
+            oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[j], oacc[t], 0, 0, 0);
+        }
+    mx_cur = tile_row_max(s_next);
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 4 * (HD / 32); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+    }
+}
+
+struct PackedParams {
+    const bf16_t* q; int64_t ldq;
+    const char* kp;              // [n_heads][n_tiles][tile bytes]
+    const char* vp;
+    bf16_t* o; int64_t ldo;
+    int n_tokens, n_heads;
+    float scale_log2e;
+};
+
+template <int HD>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_pipe_kernel(
+    const PackedParams p) {
+    constexpr int NW = 8;
+    constexpr int TILE_BYTES = BN * HD * 2;            // same for K and V tiles
+    constexpr int PER_WAVE = TILE_BYTES / 1024 / NW;   // direct-to-LDS instructions per wave per tile
+    constexpr int RING = 3;                            // K(t) lives in slot t % 3, V(t) in slot t % 3
+    __shared__ __attribute__((aligned(1024))) char sk[RING * TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char sv[RING * TILE_BYTES];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r32 = lane & 31, kh = lane >> 5;
+    const int head = blockIdx.y;
+    const int q0 = blockIdx.x * BMQ + wave * 32;
+
+    // ---- Q fragments, pre-multiplied by log2(e)/sqrt(HD) (one extra bf16 rounding of Q)
+    constexpr int QREG = QSplit<HD>::QREG;
+    const char* qstash = nullptr;
+    bf16x8 qf[QREG];
+    {
+        int qrow = q0 + r32;
+        qrow = qrow < p.n_tokens ? qrow : p.n_tokens - 1;
+        const bf16_t* qp = p.q + (int64_t)qrow * p.ldq + head * HD + 8 * kh;
+#pragma unroll
+        for (int ks = 0; ks < HD / 16; ++ks) {
+            const uint4 u = *reinterpret_cast<const uint4*>(qp + 16 * ks);
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16lo(w[e]) * p.scale_log2e, bf16hi(w[e]) * p.scale_log2e);
+            qf[ks] = __builtin_bit_cast(bf16x8, make_uint4(o[0], o[1], o[2], o[3]));
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // Q is in registers: from here on vmcnt counts tile loads only
+
+    f32x16 oacc[HD / 32];
+#pragma unroll
+    for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[t][v] = 0.0f;
+    float m_ref = 0.0f, l_run = 0.0f;
+
+    const int NT = (p.n_tokens + BN - 1) / BN;
+    const int last_valid = p.n_tokens - (NT - 1) * BN;
+    const uint32_t lane_off = (uint32_t)(wave * 1024 + lane * 16);
+    const char* kbase = p.kp + (int64_t)head * NT * TILE_BYTES;
+    const char* vbase = p.vp + (int64_t)head * NT * TILE_BYTES;
+    const uint32_t sk_addr = lds_addr_of(sk) + wave * 1024, sv_addr = lds_addr_of(sv) + wave * 1024;
+
+    // tile `t` (clamped to the last tile, so that every step issues the same number of loads and the
+    // vmcnt arithmetic below stays valid at the end of the sequence) -> ring slot `slot`
+    auto issue = [&](const char* base, uint32_t dst_addr, int t, int slot) {
+        const char* src = base + (int64_t)(t < NT ? t : NT - 1) * TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i)
+            lds_dma16(src + i * (NW * 1024), lane_off, dst_addr + slot * TILE_BYTES + i * (NW * 1024));
+    };
+
+    // ---- prologue: K(0) | K(1), V(0) | K(2), V(1); scores of tile 0 with an exact first reference
+    issue(kbase, sk_addr, 0, 0);
+    issue(kbase, sk_addr, 1, 1);
+    issue(vbase, sv_addr, 0, 0);
+    issue(kbase, sk_addr, 2, 2);
+    issue(vbase, sv_addr, 1, 1);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * PER_WAVE) : "memory");   // K(0) has landed
+    f32x16 s_a[2], s_b[2];      // score tiles ping-pong between the two halves of the unrolled loop
+    const bool ragged = last_valid < BN;
+    init_scores(s_a, 0.0f, NT == 1 && ragged, last_valid, lane);
+    scores_tile<HD>(sk, qf, qstash, s_a, lane);
+    m_ref = tile_row_max(s_a);
+    float mx_cur = 0.0f;        // row maximum of the current scores relative to m_ref
+#pragma unroll
+    for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_a[kvb][v] -= m_ref;
+
+    // step j: S(j+1) from K slot (j+1)%3, P(j) V(j) from V slot j%3; the loads of K(j+2), V(j+1) (issued one
+    // step ago) may still be in flight, those of K(j+1), V(j) (two steps ago) must have landed:
+    // s_waitcnt vmcnt(2 tiles).  After the barrier every wave is done with K(j) and V(j-1), whose slots are
+    // refilled with K(j+3) and V(j+2).
+    int ks_next = 1, vs_cur = 0;      // ring slots: (j+1)%3 and j%3
+#define CDM_ATTN_STEP(SCUR, SNEXT)                                                                              \
+    {                                                                                                           \
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER_WAVE) : "memory");                       \
+        const int k_fill = vs_cur;                              /* slot of K(j)   == j % 3     */               \
+        const int v_fill = ks_next == 2 ? 0 : ks_next + 1;      /* slot of V(j-1) == (j+2) % 3 */               \
+        issue(kbase, sk_addr, j + 3, k_fill);                                                                   \
+        issue(vbase, sv_addr, j + 2, v_fill);                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        pipe_step<HD>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, qf, qstash, SCUR, SNEXT, oacc, m_ref,  \
+                      mx_cur, l_run, lane, ragged && j + 2 == NT, last_valid);                                  \
+        vs_cur = ks_next;                                                                                       \
+        ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
+    }
+    for (int j = 0; j < NT; ++j) {
+        CDM_ATTN_STEP(s_a, s_b)
+        if (++j >= NT) break;
+        CDM_ATTN_STEP(s_b, s_a)
+    }
+#undef CDM_ATTN_STEP
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct-to-LDS write may outlive the workgroup
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / l_tot;
+    const int qrow = q0 + r32;
+    if (qrow < p.n_tokens) {
+        bf16_t* op = p.o + (int64_t)qrow * p.ldo + head * HD + 4 * kh;
+#pragma unroll
+        for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2 w;
+                w.x = pack_bf16x2(oacc[t][4 * g + 0] * inv, oacc[t][4 * g + 1] * inv);
+                w.y = pack_bf16x2(oacc[t][4 * g + 2] * inv, oacc[t][4 * g + 3] * inv);
+                *reinterpret_cast<uint2*>(op + 32 * t + 8 * g) = w;
+            }
+    }
+}
+
+// K, V [n_tokens, n_heads, HD] -> tile images Kp, Vp (see above); one workgroup per (64-key tile, head)
+template <int HD>
+__global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__ k, int64_t ldk,
+                                                      const bf16_t* __restrict__ v, int64_t ldv,
+                                                      char* __restrict__ kp, char* __restrict__ vp, int n_tokens,
+                                                      int n_tiles) {
+    __shared__ bf16_t tile[64][HD + 2];
+    constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
+    constexpr int TILE_BYTES = BN * HD * 2;
+    const int tile_idx = blockIdx.x, head = blockIdx.y;
+    const int t0 = tile_idx * 64;
+    char* kt = kp + ((int64_t)head * n_tiles + tile_idx) * TILE_BYTES;
+    char* vt = vp + ((int64_t)head * n_tiles + tile_idx) * TILE_BYTES;
+    for (int idx = threadIdx.x; idx < 64 * CPR; idx += 256) {
+        const int r = idx / CPR, ch = idx % CPR;
+        uint4 uk = make_uint4(0, 0, 0, 0), uv = uk;
+        if (t0 + r < n_tokens) {
+            uk = *reinterpret_cast<const uint4*>(k + (int64_t)(t0 + r) * ldk + head * HD + ch * 8);
+            uv = *reinterpret_cast<const uint4*>(v + (int64_t)(t0 + r) * ldv + head * HD + ch * 8);
+        }
+        *reinterpret_cast<uint4*>(kt + (ch * 64 + r) * 16) = uk;          // chunk-major K image
+        uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[r][ch * 8]);
+        dst[0] = uv.x; dst[1] = uv.y; dst[2] = uv.z; dst[3] = uv.w;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < HD * 8; idx += 256) {
+        const int row = idx % HD, c = idx / HD;                            // channel row, key chunk
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            w[e] = (uint32_t)tile[c * 8 + 2 * e][row] | ((uint32_t)tile[c * 8 + 2 * e + 1][row] << 16);
+        *reinterpret_cast<uint4*>(vt + (c * HD + row) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
 // V[n_tokens, n_heads, HD] (row stride ldv) -> Vt[n_heads][HD][n_pad], zero beyond n_tokens
 template <int HD>
 __global__ __launch_bounds__(256) void transpose_v_kernel(const bf16_t* __restrict__ v, int64_t ldv,
@@ -302,21 +625,15 @@ __global__ __launch_bounds__(256) void transpose_v_kernel(const bf16_t* __restri
 }
 
 inline int64_t pad_tokens(int64_t n) { return (n + BN - 1) / BN * BN; }
+inline int64_t image_bytes(int64_t n_tokens, int n_heads, int head_dim) {      // one packed tensor
+    return pad_tokens(n_tokens) * n_heads * head_dim * 2;
+}
 
 template <int HD, int QSUB, int NW>
 void launch_attn(const AttnParams& p, hipStream_t st) {
     dim3 grid((p.n_tokens + BMQ - 1) / BMQ, p.n_heads);
     attn_fwd_kernel<HD, QSUB, NW><<<grid, NW * 64, 0, st>>>(p);
 }
-
-}  // namespace
-
-extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
-    if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0) return 0;
-    return pad_tokens(n_tokens) * n_heads * head_dim * 2;
-}
-
-namespace {
 
 int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
     CDM_REQUIRE(n_tokens >= 0 && n_heads > 0, CDM_ERR_BAD_ARG, "%s: bad sizes", who);
@@ -327,61 +644,65 @@ int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, in
 
 }  // namespace
 
-extern "C" int32_t cdm_transpose_v_bf16(const void* v, int64_t ldv, void* vt, int64_t vt_bytes, int64_t n_tokens,
-                                        int32_t n_heads, int32_t head_dim, void* stream) {
-    CDM_REQUIRE(v && vt, CDM_ERR_BAD_ARG, "transpose_v: null pointer");
-    int32_t rc = check_attn_common("transpose_v", n_tokens, n_heads, head_dim);
-    if (rc) return rc;
-    CDM_REQUIRE(ldv >= (int64_t)n_heads * head_dim, CDM_ERR_BAD_ARG, "transpose_v: row stride smaller than n_heads*head_dim");
-    CDM_REQUIRE(cdm_aligned16(v) && cdm_aligned16(vt) && ldv % 8 == 0, CDM_ERR_BAD_ALIGN,
-                "transpose_v: pointers/strides must be 16-byte aligned");
-    const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim);
-    CDM_REQUIRE(vt_bytes >= need, CDM_ERR_BAD_ARG, "transpose_v: output of at least %lld bytes required", (long long)need);
-    if (n_tokens == 0) return CDM_OK;
-    if ((rc = cdm_require_device())) return rc;
-    const int n_pad = (int)pad_tokens(n_tokens);
-    dim3 tgrid(n_pad / 64, n_heads);
-    hipStream_t st = (hipStream_t)stream;
-    if (head_dim == 128)
-        transpose_v_kernel<128><<<tgrid, 256, 0, st>>>((const bf16_t*)v, ldv, (bf16_t*)vt, (int)n_tokens, n_pad);
-    else
-        transpose_v_kernel<64><<<tgrid, 256, 0, st>>>((const bf16_t*)v, ldv, (bf16_t*)vt, (int)n_tokens, n_pad);
-    return cdm_check_launch("transpose_v");
+// workspace = [Kp | Vp | V^T]: the two tile images of the pipelined kernel, then the plain per-head
+// transpose of V that the non-pipelined variants read
+extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
+    if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0) return 0;
+    return 3 * image_bytes(n_tokens, n_heads, head_dim);
 }
 
-extern "C" int32_t cdm_attn_fwd_vt_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
-                                        void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
-                                        void* stream) {
-    CDM_REQUIRE(q && k && vt && o, CDM_ERR_BAD_ARG, "attn_fwd: null pointer");
-    int32_t rc = check_attn_common("attn_fwd", n_tokens, n_heads, head_dim);
+extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, void* workspace,
+                                         int64_t workspace_bytes, int64_t n_tokens, int32_t n_heads,
+                                         int32_t head_dim, void* stream) {
+    CDM_REQUIRE(k && v && workspace, CDM_ERR_BAD_ARG, "attn_pack_kv: null pointer");
+    int32_t rc = check_attn_common("attn_pack_kv", n_tokens, n_heads, head_dim);
     if (rc) return rc;
     const int64_t d = (int64_t)n_heads * head_dim;
-    CDM_REQUIRE(ldq >= d && ldk >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd: row stride smaller than n_heads*head_dim");
-    CDM_REQUIRE(ldk * 64 * 2 < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd: ldk out of range");
-    CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(k) && cdm_aligned16(vt) && cdm_aligned16(o) && ldq % 8 == 0 &&
-                    ldk % 8 == 0 && ldo % 4 == 0,
-                CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
+    CDM_REQUIRE(ldk >= d && ldv >= d, CDM_ERR_BAD_ARG, "attn_pack_kv: row stride smaller than n_heads*head_dim");
+    CDM_REQUIRE(cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(workspace) && ldk % 8 == 0 && ldv % 8 == 0,
+                CDM_ERR_BAD_ALIGN, "attn_pack_kv: pointers/strides must be 16-byte aligned");
+    const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim);
+    CDM_REQUIRE(workspace_bytes >= need, CDM_ERR_BAD_ARG, "attn_pack_kv: workspace of at least %lld bytes required",
+                (long long)need);
     if (n_tokens == 0) return CDM_OK;
     if ((rc = cdm_require_device())) return rc;
-    AttnParams p;
-    p.q = (const bf16_t*)q; p.ldq = ldq;
-    p.k = (const bf16_t*)k; p.ldk = ldk;
-    p.vt = (const bf16_t*)vt;
-    p.o = (bf16_t*)o; p.ldo = ldo;
-    p.n_tokens = (int)n_tokens; p.n_pad = (int)pad_tokens(n_tokens); p.n_heads = n_heads;
-    p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
+    const int n_tiles = (int)(pad_tokens(n_tokens) / BN);
+    const int64_t img = image_bytes(n_tokens, n_heads, head_dim);
+    char* ws = (char*)workspace;
+    dim3 grid(n_tiles, n_heads);
     hipStream_t st = (hipStream_t)stream;
-    const int variant = cdm_get_variant(0);
-    // variant 0: 8 waves x 32 query rows (two waves per SIMD overlap softmax with MFMA);
-    // variant 1: 4 waves x 64 query rows (half the LDS traffic per flop, one wave per SIMD)
-    if (head_dim == 128) {
-        if (variant == 1) launch_attn<128, 2, 4>(p, st);
-        else launch_attn<128, 1, 8>(p, st);
-    } else {
-        if (variant == 1) launch_attn<64, 2, 4>(p, st);
-        else launch_attn<64, 1, 8>(p, st);
-    }
-    return cdm_check_launch("attn_fwd");
+    if (head_dim == 128)
+        pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, ws, ws + img,
+                                                  (int)n_tokens, n_tiles);
+    else
+        pack_kv_kernel<64><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, ws, ws + img,
+                                                 (int)n_tokens, n_tiles);
+    return cdm_check_launch("attn_pack_kv");
+}
+
+extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const void* workspace, void* o, int64_t ldo,
+                                            int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream) {
+    CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
+    int32_t rc = check_attn_common("attn_fwd_packed", n_tokens, n_heads, head_dim);
+    if (rc) return rc;
+    const int64_t d = (int64_t)n_heads * head_dim;
+    CDM_REQUIRE(ldq >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd_packed: row stride smaller than n_heads*head_dim");
+    CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(workspace) && cdm_aligned16(o) && ldq % 8 == 0 && ldo % 4 == 0,
+                CDM_ERR_BAD_ALIGN, "attn_fwd_packed: pointers/strides must be 16-byte aligned");
+    if (n_tokens == 0) return CDM_OK;
+    if ((rc = cdm_require_device())) return rc;
+    const int64_t img = image_bytes(n_tokens, n_heads, head_dim);
+    PackedParams p;
+    p.q = (const bf16_t*)q; p.ldq = ldq;
+    p.kp = (const char*)workspace; p.vp = (const char*)workspace + img;
+    p.o = (bf16_t*)o; p.ldo = ldo;
+    p.n_tokens = (int)n_tokens; p.n_heads = n_heads;
+    p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
+    dim3 grid((unsigned)((n_tokens + BMQ - 1) / BMQ), n_heads);
+    hipStream_t st = (hipStream_t)stream;
+    if (head_dim == 128) attn_fwd_pipe_kernel<128><<<grid, 512, 0, st>>>(p);
+    else attn_fwd_pipe_kernel<64><<<grid, 512, 0, st>>>(p);
+    return cdm_check_launch("attn_fwd_packed");
 }
 
 extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
@@ -394,13 +715,42 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
     const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim);
     CDM_REQUIRE(workspace && cdm_aligned16(workspace) && workspace_bytes >= need, CDM_ERR_BAD_ARG,
                 "attn_fwd: workspace of at least %lld bytes required", (long long)need);
-    // validate the second stage's arguments before the first stage is enqueued
+    // validate everything before the first stage is enqueued
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldq >= d && ldk >= d && ldv >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd: row stride smaller than n_heads*head_dim");
     CDM_REQUIRE(ldk * 64 * 2 < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd: ldk out of range");
     CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(o) && ldq % 8 == 0 &&
                     ldk % 8 == 0 && ldv % 8 == 0 && ldo % 4 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
-    if ((rc = cdm_transpose_v_bf16(v, ldv, workspace, workspace_bytes, n_tokens, n_heads, head_dim, stream))) return rc;
-    return cdm_attn_fwd_vt_bf16(q, ldq, k, ldk, workspace, o, ldo, n_tokens, n_heads, head_dim, stream);
+    if ((rc = cdm_require_device())) return rc;
+    const int variant = cdm_get_variant(0);
+    if (variant == 0) {
+        if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, workspace, workspace_bytes, n_tokens, n_heads, head_dim, stream)))
+            return rc;
+        return cdm_attn_fwd_packed_bf16(q, ldq, workspace, o, ldo, n_tokens, n_heads, head_dim, stream);
+    }
+    // measurement variants (non-pipelined kernel on row-major K and per-head V^T):
+    // 1 = 8 waves x 32 query rows, 2 = 4 waves x 64 query rows
+    hipStream_t st = (hipStream_t)stream;
+    const int n_pad = (int)pad_tokens(n_tokens);
+    bf16_t* vt = (bf16_t*)((char*)workspace + 2 * image_bytes(n_tokens, n_heads, head_dim));
+    dim3 tgrid(n_pad / 64, n_heads);
+    if (head_dim == 128) transpose_v_kernel<128><<<tgrid, 256, 0, st>>>((const bf16_t*)v, ldv, vt, (int)n_tokens, n_pad);
+    else transpose_v_kernel<64><<<tgrid, 256, 0, st>>>((const bf16_t*)v, ldv, vt, (int)n_tokens, n_pad);
+    if ((rc = cdm_check_launch("attn_fwd(transpose_v)"))) return rc;
+    AttnParams p;
+    p.q = (const bf16_t*)q; p.ldq = ldq;
+    p.k = (const bf16_t*)k; p.ldk = ldk;
+    p.vt = vt;
+    p.o = (bf16_t*)o; p.ldo = ldo;
+    p.n_tokens = (int)n_tokens; p.n_pad = n_pad; p.n_heads = n_heads;
+    p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
+    if (head_dim == 128) {
+        if (variant == 2) launch_attn<128, 2, 4>(p, st);
+        else launch_attn<128, 1, 8>(p, st);
+    } else {
+        if (variant == 2) launch_attn<64, 2, 4>(p, st);
+        else launch_attn<64, 1, 8>(p, st);
+    }
+    return cdm_check_launch("attn_fwd");
 }

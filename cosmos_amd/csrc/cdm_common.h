@@ -64,3 +64,20 @@ __device__ __forceinline__ float wave_max(float v) {
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
     return v;
 }
+
+// One 16-byte-per-lane direct-to-LDS load, written as inline assembly so that the compiler's wait-count
+// insertion does not see an LDS write it would have to guard conservatively across a loop back-edge (it would
+// put s_waitcnt vmcnt(0) in front of fragment reads and drain a multi-stage pipeline).  Every wait on these
+// loads is therefore an explicit s_waitcnt vmcnt(n) written by the kernel that issued them.  M0 = LDS byte address of the wave's
+// 1 KB destination; one wait state is required between the M0 write and the load.
+__device__ __forceinline__ void lds_dma16(const char* uniform_base, uint32_t lane_offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(lane_offset), "s"(uniform_base)
+                 : "memory", "m0");
+}
+
+__device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)p;
+}
+

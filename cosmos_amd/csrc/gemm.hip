@@ -36,6 +36,7 @@ struct GemmParams {
     const float* cos; const float* sin;
     int rope_cols, head_dim;
     int tiles_m, tiles_n;
+    int k_rotate;        // 1: each tile starts its K walk at its own offset
 };
 
 // chunk swizzle: 16-byte chunk c of tile row r lives at chunk position c ^ swz(r)
@@ -108,85 +109,10 @@ __device__ __forceinline__ void issue_loads(const char* abase, const char* wbase
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
 
+// ---- epilogue shared by both pipelines
 template <int EPI, bool FP8>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(1024))) char sa0[kTileBytes];
-    __shared__ __attribute__((aligned(1024))) char sb0[kTileBytes];
-    __shared__ __attribute__((aligned(1024))) char sa1[kTileBytes];
-    __shared__ __attribute__((aligned(1024))) char sb1[kTileBytes];
-
-    // ---- XCD-aware tile assignment
-    const int total = p.tiles_m * p.tiles_n;
-    const int per_xcd = (total + 7) >> 3;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
-    constexpr int GM = 8;
-    const int group = logical / (GM * p.tiles_n);
-    const int first_m = group * GM;
-    const int gsz = (p.tiles_m - first_m) < GM ? (p.tiles_m - first_m) : GM;
-    const int in_group = logical - group * GM * p.tiles_n;
-    const int tm = first_m + in_group % gsz;
-    const int tn = in_group / gsz;
-
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = tm * BM;
-    const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
-
-    // ---- per-lane byte offsets (relative to the tile's first row) of the 8 + 8 loads of one k-tile
-    uint32_t oa[8], ob[8];
-    uint32_t w2mask = 0;     // bit i set: load i of this wave reads W2 (up_proj rows of a SWIGLU tile)
-    int nb0 = n0;            // first W row of the tile
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int row = (i * 4 + wave) * 8 + (lane >> 3);   // tile row this lane feeds
-        const int chunk = (lane & 7) ^ swz(row);            // source chunk that belongs at position lane&7
-        int am = row;
-        am = (m0 + am) < p.M ? am : p.M - 1 - m0;
-        oa[i] = (uint32_t)(am * (int)p.lda + chunk * 16);
-        int bn;
-        if (EPI == CDM_EPI_SWIGLU) {
-            // 64-row groups of the tile alternate gate / up: [g 0-63 | u 0-63 | g 64-127 | u 64-127]
-            const int grp = ((i * 4 + wave) * 8) >> 6;       // wave-uniform
-            if (grp & 1) w2mask |= 1u << i;
-            bn = (grp >> 1) * 64 + (row & 63);
-        } else {
-            bn = row;
-        }
-        bn = (nb0 + bn) < p.N ? bn : p.N - 1 - nb0;
-        ob[i] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
-    }
-    const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
-    const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)nb0 * p.ldw;
-    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)nb0 * p.ldw : wbase;
-
-    f32x16 acc[4][4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
-
-    const int KT = p.K / (FP8 ? 128 : 64);   // k-tiles of 128 bytes; the host guarantees an even count
-    issue_loads(abase, wbase, w2base, oa, ob, w2mask, sa0, sb0, wave);
-    for (int kt = 0; kt < KT; kt += 2) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        issue_loads(abase + (kt + 1) * 128, wbase + (kt + 1) * 128, w2base + (kt + 1) * 128, oa, ob, w2mask, sa1, sb1,
-                    wave);
-        __builtin_amdgcn_sched_barrier(0);      // keep the prefetch at the top of the stage
-        compute_stage<FP8>(sa0, sb0, acc, wm, wn, lane);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (kt + 2 < KT)
-            issue_loads(abase + (kt + 2) * 128, wbase + (kt + 2) * 128, w2base + (kt + 2) * 128, oa, ob, w2mask, sa0,
-                        sb0, wave);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_stage<FP8>(sa1, sb1, acc, wm, wn, lane);
-    }
-
+__device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4], int m0, int n0, int wm, int wn,
+                                         int lane) {
     // ---- epilogue: accumulator (mi, ni, v) is row 8*(v/4) + 4*(lane/32) + v%4, column lane%32 of its 32x32 block
     const int r32 = lane & 31, kh = lane >> 5;
     const int row_base = m0 + wm * 128 + 4 * kh;
@@ -280,6 +206,253 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
 }
 
+template <int EPI, bool FP8>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(1024))) char sa0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char sb0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char sa1[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char sb1[kTileBytes];
+
+    // ---- XCD-aware tile assignment
+    const int total = p.tiles_m * p.tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    constexpr int GM = 8;
+    const int group = logical / (GM * p.tiles_n);
+    const int first_m = group * GM;
+    const int gsz = (p.tiles_m - first_m) < GM ? (p.tiles_m - first_m) : GM;
+    const int in_group = logical - group * GM * p.tiles_n;
+    const int tm = first_m + in_group % gsz;
+    const int tn = in_group / gsz;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = tm * BM;
+    const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
+
+    // ---- per-lane byte offsets (relative to the tile's first row) of the 8 + 8 loads of one k-tile
+    uint32_t oa[8], ob[8];
+    uint32_t w2mask = 0;     // bit i set: load i of this wave reads W2 (up_proj rows of a SWIGLU tile)
+    int nb0 = n0;            // first W row of the tile
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = (i * 4 + wave) * 8 + (lane >> 3);   // tile row this lane feeds
+        const int chunk = (lane & 7) ^ swz(row);            // source chunk that belongs at position lane&7
+        int am = row;
+        am = (m0 + am) < p.M ? am : p.M - 1 - m0;
+        oa[i] = (uint32_t)(am * (int)p.lda + chunk * 16);
+        int bn;
+        if (EPI == CDM_EPI_SWIGLU) {
+            // 64-row groups of the tile alternate gate / up: [g 0-63 | u 0-63 | g 64-127 | u 64-127]
+            const int grp = ((i * 4 + wave) * 8) >> 6;       // wave-uniform
+            if (grp & 1) w2mask |= 1u << i;
+            bn = (grp >> 1) * 64 + (row & 63);
+        } else {
+            bn = row;
+        }
+        bn = (nb0 + bn) < p.N ? bn : p.N - 1 - nb0;
+        ob[i] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
+    }
+    const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
+    const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)nb0 * p.ldw;
+    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)nb0 * p.ldw : wbase;
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+    const int KT = p.K / (FP8 ? 128 : 64);   // k-tiles of 128 bytes; the host guarantees an even count
+    issue_loads(abase, wbase, w2base, oa, ob, w2mask, sa0, sb0, wave);
+    for (int kt = 0; kt < KT; kt += 2) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        issue_loads(abase + (kt + 1) * 128, wbase + (kt + 1) * 128, w2base + (kt + 1) * 128, oa, ob, w2mask, sa1, sb1,
+                    wave);
+        __builtin_amdgcn_sched_barrier(0);      // keep the prefetch at the top of the stage
+        compute_stage<FP8>(sa0, sb0, acc, wm, wn, lane);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (kt + 2 < KT)
+            issue_loads(abase + (kt + 2) * 128, wbase + (kt + 2) * 128, w2base + (kt + 2) * 128, oa, ob, w2mask, sa0,
+                        sb0, wave);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_stage<FP8>(sa1, sb1, acc, wm, wn, lane);
+    }
+
+    epilogue<EPI, FP8>(p, acc, m0, n0, wm, wn, lane);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Deep pipeline: same 256x256 tile and wave layout, but k-tiles of 64 BYTES and FOUR LDS stages
+// (4 x 32 KB), so the loads of k-tiles t+1 .. t+3 are in flight while k-tile t is multiplied
+// (about three stage times of latency tolerance instead of one).  A wave waits only for its own
+// loads of tile t (s_waitcnt vmcnt(16): the 2 x 8 younger loads may stay outstanding) before the
+// workgroup barrier.  Rows are 64 bytes = 4 chunks; chunk c of row r sits at position
+// c ^ (((r >> 1) ^ (r >> 3)) & 3), which keeps 8 and 16 consecutive lanes on distinct banks.
+// ---------------------------------------------------------------------------------------------
+constexpr int kStageBytes4 = BM * 64;   // 16 KB per operand per stage
+
+__device__ __forceinline__ int swz4(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
+
+__device__ __forceinline__ bf16x8 lds_frag4(const char* tile, int row, int chunk) {
+    return *reinterpret_cast<const bf16x8*>(tile + row * 64 + ((chunk ^ swz4(row)) << 4));
+}
+
+template <bool FP8>
+__device__ __forceinline__ void compute_stage4(const char* sa, const char* sb, f32x16 (&acc)[4][4], int wm, int wn,
+                                               int lane) {
+    const int r32 = lane & 31, kh = lane >> 5;
+    if (!FP8) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {     // 2 x 16 bf16 = 64 bytes
+            bf16x8 af[4], bfr[4];
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) af[mi] = lds_frag4(sa, wm * 128 + mi * 32 + r32, 2 * ks + kh);
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) bfr[ni] = lds_frag4(sb, wn * 128 + ni * 32 + r32, 2 * ks + kh);
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 4; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0);
+        }
+    } else {
+        i32x8 af[4], bfr[4];                 // 64 e4m3: one 32x32x64 MFMA step
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+            const int4 l4 = __builtin_bit_cast(int4, lds_frag4(sa, wm * 128 + mi * 32 + r32, 2 * kh));
+            const int4 h4 = __builtin_bit_cast(int4, lds_frag4(sa, wm * 128 + mi * 32 + r32, 2 * kh + 1));
+            af[mi] = i32x8{l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
+        }
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) {
+            const int4 l4 = __builtin_bit_cast(int4, lds_frag4(sb, wn * 128 + ni * 32 + r32, 2 * kh));
+            const int4 h4 = __builtin_bit_cast(int4, lds_frag4(sb, wn * 128 + ni * 32 + r32, 2 * kh + 1));
+            bfr[ni] = i32x8{l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
+        }
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0,
+                                                                              0x7f7f7f7f, 0, 0x7f7f7f7f);
+    }
+}
+
+__device__ __forceinline__ void issue_loads4(const char* abase, const char* wbase, const char* w2base,
+                                             const uint32_t (&oa)[4], const uint32_t (&ob)[4], uint32_t w2mask,
+                                             char* sa, char* sb, int wave) {
+    const uint32_t la = lds_addr_of(sa) + wave * 1024, lb = lds_addr_of(sb) + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        lds_dma16(abase, oa[i], la + i * 4096);
+        const char* wb = ((w2mask >> i) & 1u) ? w2base : wbase;   // wave-uniform choice
+        lds_dma16(wb, ob[i], lb + i * 4096);
+    }
+}
+
+template <int EPI, bool FP8>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel4(const GemmParams p) {
+    __shared__ __attribute__((aligned(1024))) char sa0[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sb0[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sa1[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sb1[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sa2[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sb2[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sa3[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char sb3[kStageBytes4];
+
+    const int total = p.tiles_m * p.tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    constexpr int GM = 8;
+    const int group = logical / (GM * p.tiles_n);
+    const int first_m = group * GM;
+    const int gsz = (p.tiles_m - first_m) < GM ? (p.tiles_m - first_m) : GM;
+    const int in_group = logical - group * GM * p.tiles_n;
+    const int tm = first_m + in_group % gsz;
+    const int tn = in_group / gsz;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = tm * BM;
+    const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
+
+    // per-lane byte offsets of the 4 + 4 loads of one k-tile (each instruction = 16 tile rows of 64 bytes)
+    uint32_t oa[4], ob[4];
+    uint32_t w2mask = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = (i * 4 + wave) * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ swz4(row);
+        int am = row;
+        am = (m0 + am) < p.M ? am : p.M - 1 - m0;
+        oa[i] = (uint32_t)(am * (int)p.lda + chunk * 16);
+        int bn;
+        if (EPI == CDM_EPI_SWIGLU) {
+            const int grp = ((i * 4 + wave) * 16) >> 6;      // wave-uniform
+            if (grp & 1) w2mask |= 1u << i;
+            bn = (grp >> 1) * 64 + (row & 63);
+        } else {
+            bn = row;
+        }
+        bn = (n0 + bn) < p.N ? bn : p.N - 1 - n0;
+        ob[i] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
+    }
+    const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
+    const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)n0 * p.ldw;
+    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)n0 * p.ldw : wbase;
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+    const int KT = p.K / (FP8 ? 64 : 32);   // k-tiles of 64 bytes; a multiple of 4 (host-checked)
+    // Every tile walks K from its own starting point (the sum over k is order-free).  With power-of-two row
+    // strides all 256 rows of a k-tile sit at the same offset modulo the stride, so workgroups marching
+    // through K in lockstep would all hit the same L2 / memory channels at the same time.
+    const int rot = p.k_rotate ? ((logical * 10) % KT) & ~1 : 0;
+    auto koff = [&](int t) {          // byte offset of the t-th k-tile this workgroup processes
+        int kk = t + rot;
+        kk = kk >= KT ? kk - KT : kk;
+        return kk * 64;
+    };
+    issue_loads4(abase + koff(0), wbase + koff(0), w2base + koff(0), oa, ob, w2mask, sa0, sb0, wave);
+    issue_loads4(abase + koff(1), wbase + koff(1), w2base + koff(1), oa, ob, w2mask, sa1, sb1, wave);
+    issue_loads4(abase + koff(2), wbase + koff(2), w2base + koff(2), oa, ob, w2mask, sa2, sb2, wave);
+    // stage t: wait for tile t (younger tiles stay in flight), barrier, refill the buffer freed by tile t-1
+#define CDM_STAGE(T, SA, SB, SA_FILL, SB_FILL)                                                              \
+    if ((T) + 2 < KT) asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");                        \
+    else if ((T) + 1 < KT) asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");                    \
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");                                      \
+    if ((T) + 3 < KT) {                                                                                     \
+        const int ko = koff((T) + 3);                                                                       \
+        issue_loads4(abase + ko, wbase + ko, w2base + ko, oa, ob, w2mask, SA_FILL, SB_FILL, wave);          \
+    }                                                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                      \
+    compute_stage4<FP8>(SA, SB, acc, wm, wn, lane);
+    for (int kt = 0; kt < KT; kt += 4) {
+        CDM_STAGE(kt, sa0, sb0, sa3, sb3)
+        CDM_STAGE(kt + 1, sa1, sb1, sa0, sb0)
+        CDM_STAGE(kt + 2, sa2, sb2, sa1, sb1)
+        CDM_STAGE(kt + 3, sa3, sb3, sa2, sb2)
+    }
+#undef CDM_STAGE
+    epilogue<EPI, FP8>(p, acc, m0, n0, wm, wn, lane);
+}
+
 // esize = bytes per operand element (2 = bf16, 1 = e4m3); strides in elements
 int32_t validate(const char* who, int esize, const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2,
                  void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epi, const void* R, int64_t ldr,
@@ -320,12 +493,20 @@ int32_t run(GemmParams& p, int64_t M, int64_t N, int32_t epilogue, hipStream_t s
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
+    // variant 0 = four-stage pipeline with per-tile K rotation (default); 1 = two-stage; 2 = four-stage, no rotation
+    const int variant = cdm_get_variant(1);
+    const bool deep = variant != 1;
+    p.k_rotate = variant == 0;
+#define CDM_LAUNCH(E)                                                         \
+    if (deep) gemm_kernel4<E, FP8><<<grid, kThreads, 0, st>>>(p);             \
+    else gemm_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p)
     switch (epilogue) {
-        case CDM_EPI_NONE: gemm_kernel<CDM_EPI_NONE, FP8><<<grid, kThreads, 0, st>>>(p); break;
-        case CDM_EPI_SWIGLU: gemm_kernel<CDM_EPI_SWIGLU, FP8><<<grid, kThreads, 0, st>>>(p); break;
-        case CDM_EPI_GATE_RESIDUAL: gemm_kernel<CDM_EPI_GATE_RESIDUAL, FP8><<<grid, kThreads, 0, st>>>(p); break;
-        default: gemm_kernel<CDM_EPI_ROPE_QK, FP8><<<grid, kThreads, 0, st>>>(p); break;
+        case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;
+        case CDM_EPI_SWIGLU: CDM_LAUNCH(CDM_EPI_SWIGLU); break;
+        case CDM_EPI_GATE_RESIDUAL: CDM_LAUNCH(CDM_EPI_GATE_RESIDUAL); break;
+        default: CDM_LAUNCH(CDM_EPI_ROPE_QK); break;
     }
+#undef CDM_LAUNCH
     return cdm_check_launch(who);
 }
 

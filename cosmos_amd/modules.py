@@ -54,7 +54,15 @@ class Workspace:
 class DMAttnProcessor:
     """Attention processor: per-branch QKV projection with mRoPE in the GEMM epilogue, ONE shared full
     attention over the joint sequence, per-branch output projection (optionally fused with the gated
-    residual)."""
+    residual).
+
+    ``rope_in_gemm_epilogue`` selects where mRoPE is applied: inside the QKV GEMM epilogue (on the fp32
+    accumulators) or by the streaming in-place kernel right after a plain QKV GEMM.  The second is the default:
+    the rotating epilogue currently costs more GEMM time than the extra 8*N*d bytes of the streaming pass.
+    """
+
+    def __init__(self, rope_in_gemm_epilogue: bool = False):
+        self.rope_in_gemm_epilogue = rope_in_gemm_epilogue
 
     def __call__(self, attn: "DMAttention", hidden_states: torch.Tensor,
                  encoder_hidden_states: Optional[torch.Tensor] = None, attention_mask: Optional[torch.Tensor] = None,
@@ -87,8 +95,12 @@ class DMAttnProcessor:
         qkv = ws.qkv if ws is not None else torch.empty((n, 3 * d), dtype=torch.bfloat16, device=x.device)
         o = ws.attn_out if ws is not None else torch.empty((n, d), dtype=torch.bfloat16, device=x.device)
 
-        attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
-                     rope_cols=2 * d, head_dim=attn.head_dim)
+        if self.rope_in_gemm_epilogue:
+            attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
+                         rope_cols=2 * d, head_dim=attn.head_dim)
+        else:
+            attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
+            ops.mrope_qk_(qkv[:, :d], qkv[:, d:2 * d], cos, sin, attn.n_heads, attn.head_dim)
         ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], attn.n_heads, attn.head_dim, out=o,
                       workspace=ws.attn_ws if ws is not None else None)
         if attn.fp8:

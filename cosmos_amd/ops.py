@@ -45,8 +45,13 @@ def _f32vec(t: Optional[torch.Tensor], name: str, n: int) -> int:
     return _chk(t.reshape(-1), name)
 
 
+_ATTN_VARIANT = [0]
+
+
 def set_variant(op: str, variant: int) -> int:
     lib = _lib.load()
+    if op == "attn":
+        _ATTN_VARIANT[0] = int(variant)
     prev = lib.cdm_set_variant(op.encode(), int(variant))
     if prev < 0:
         raise RuntimeError(f"set_variant failed: {_lib.last_error()}")
@@ -214,20 +219,20 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
     qp, kp, vp = _chk(q, "q", torch.bfloat16, 2), _chk(k, "k", torch.bfloat16, 2), _chk(v, "v", torch.bfloat16, 2)
     op, wp = _chk(out, "out", torch.bfloat16, 2), _chk(workspace, "workspace", torch.uint8, 1)
-    if _ATTN_TIMER is None:
+    if _ATTN_TIMER is None or _ATTN_VARIANT[0] != 0:
         rc = lib.cdm_attn_fwd_bf16(qp, q.stride(0), kp, k.stride(0), vp, v.stride(0), op, out.stride(0), n, n_heads,
                                    head_dim, wp, workspace.numel(), _stream())
         _lib.check(rc, "cdm_attn_fwd_bf16")
         return out
     # timed form: the same two stages, with HIP events around the attention kernel alone
-    rc = lib.cdm_transpose_v_bf16(vp, v.stride(0), wp, workspace.numel(), n, n_heads, head_dim, _stream())
-    _lib.check(rc, "cdm_transpose_v_bf16")
+    rc = lib.cdm_attn_pack_kv_bf16(kp, k.stride(0), vp, v.stride(0), wp, workspace.numel(), n, n_heads, head_dim,
+                                   _stream())
+    _lib.check(rc, "cdm_attn_pack_kv_bf16")
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    rc = lib.cdm_attn_fwd_vt_bf16(qp, q.stride(0), kp, k.stride(0), wp, op, out.stride(0), n, n_heads, head_dim,
-                                  _stream())
+    rc = lib.cdm_attn_fwd_packed_bf16(qp, q.stride(0), wp, op, out.stride(0), n, n_heads, head_dim, _stream())
     e1.record()
-    _lib.check(rc, "cdm_attn_fwd_vt_bf16")
+    _lib.check(rc, "cdm_attn_fwd_packed_bf16")
     _ATTN_TIMER.append((e0, e1))
     return out
 

@@ -133,8 +133,8 @@ int32_t cdm_mrope_qk_bf16(void* q, int64_t ldq, void* k, int64_t ldk, const floa
  * models/qwen3_vl/modeling_qwen3_vl.py:171-193, fp32 softmax).
  *   O = softmax(Q K^T / sqrt(head_dim)) V per head, no mask.
  *   q, k, v: [n_tokens, n_heads, head_dim] with row strides ldq, ldk, ldv; o: [n_tokens, n_heads*head_dim] (ldo).
- *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds V transposed
- *   per head); its contents are undefined afterwards.
+ *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds K and V re-laid
+ *   out as 64-key tile images); its contents are undefined afterwards.
  * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
  */
 int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim);
@@ -143,16 +143,16 @@ int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk
                           void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
- * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first
- * V[n_tokens, n_heads, head_dim] -> vt[n_heads][head_dim][n_tokens rounded up to 64] (zero padded;
- * vt_bytes >= cdm_attn_workspace_bytes), then the attention kernel proper reading vt.  A caller that
- * times or profiles the attention kernel alone, or that keeps V transposed across calls, uses these.
+ * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first K and V
+ * are packed into the workspace as tile images (a streaming pass), then the attention kernel proper
+ * reads Q and the workspace.  A caller that times or profiles the attention kernel alone, or that
+ * reuses packed K/V across calls, uses these.
  */
-int32_t cdm_transpose_v_bf16(const void* v, int64_t ldv, void* vt, int64_t vt_bytes, int64_t n_tokens,
-                             int32_t n_heads, int32_t head_dim, void* stream);
-int32_t cdm_attn_fwd_vt_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* vt,
-                             void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
-                             void* stream);
+int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, void* workspace,
+                              int64_t workspace_bytes, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
+                              void* stream);
+int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const void* workspace, void* o, int64_t ldo,
+                                 int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream);
 
 /*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each

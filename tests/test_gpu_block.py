@@ -54,6 +54,20 @@ def test_c0_single_block_parity():
     assert_close(y2.float().cpu() - xr, want2 - xr, 0.999, BF16_REL, "C0 block update")
 
 
+def test_rope_epilogue_and_streaming_rope_agree():
+    from cosmos_amd import DMAttnProcessor
+    cfg = DMConfig("t", 256, 2, 128, 512, 1, (2, 4, 8), n_text=8)
+    blk = make_block(cfg, 5)
+    g = torch.Generator().manual_seed(5)
+    x, _ = rand_bf16((cfg.n_tokens, 256), g)
+    temb, _ = rand_bf16((256,), g)
+    st = DMStack(cfg, device=dev())
+    y1 = blk(x, temb, st.rotary(dev()), st.segments())
+    blk.attn.set_processor(DMAttnProcessor(rope_in_gemm_epilogue=True))
+    y2 = blk(x, temb, st.rotary(dev()), st.segments())
+    assert_close(y2, y1.float().cpu(), 0.99999, 4e-3, "rope placement")
+
+
 def test_block_gate_zero_is_identity():
     cfg = DMConfig("t", 256, 2, 128, 512, 1, (2, 4, 8))
     blk = make_block(cfg, 3)

@@ -67,13 +67,19 @@ def test_mrope_standalone(hd, H, sections):
 
 
 # ------------------------------------------------------------------ GEMM
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (8, 8, 128), (300, 264, 256), (1024, 3072, 1024), (515, 1000, 384)])
-def test_gemm_plain(M, N, K):
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (8, 8, 128), (300, 264, 256), (1024, 3072, 1024), (515, 1000, 384),
+                                   (257, 520, 4096)])
+def test_gemm_plain(M, N, K, variant):
     g = gen(M + N + K)
     a, ar = rand_bf16((M, K), g)
     w, wr = rand_bf16((N, K), g, 0.05)
-    c = ops.gemm(a, w)
-    assert_close(c, ar @ wr.t(), 0.99999, 6e-3, f"gemm {M}x{N}x{K}")
+    prev = ops.set_variant("gemm", variant)
+    try:
+        c = ops.gemm(a, w)
+    finally:
+        ops.set_variant("gemm", prev)
+    assert_close(c, ar @ wr.t(), 0.99999, 6e-3, f"gemm {M}x{N}x{K} variant={variant}")
 
 
 def test_gemm_strided_views_and_determinism():
@@ -148,8 +154,9 @@ def test_grouped_gemm_three_segments():
 
 
 # ------------------------------------------------------------------ attention
-@pytest.mark.parametrize("variant", [0, 1])
-@pytest.mark.parametrize("n,H,hd", [(64, 2, 64), (256, 1, 128), (1000, 3, 128), (321, 2, 64), (1, 1, 128), (130, 2, 128)])
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("n,H,hd", [(64, 2, 64), (256, 1, 128), (1000, 3, 128), (321, 2, 64), (1, 1, 128), (130, 2, 128), (65, 1, 64),
+                                    (128, 2, 128), (191, 1, 128), (192, 1, 128), (577, 2, 128)])
 def test_attention_vs_oracle(n, H, hd, variant):
     g = gen(n + H + hd)
     d = H * hd
