@@ -131,7 +131,7 @@ def main():
                                f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
                    "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant},
-        "roofline": {"bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4), "traffic": None,
                      "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},
         "extra": {"ms_per_block": round(ms_per_step / cfg.n_blocks, 3),

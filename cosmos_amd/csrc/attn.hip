@@ -294,52 +294,51 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
 // ---------------------------------------------------------------------------------------------
 constexpr float kGrowLog2 = 4.0f;
 
-// Q fragments 0..QREG-1 stay in registers; the others are parked in a per-lane LDS slot (each lane re-reads
-// exactly the 16 bytes it wrote, so no barrier is involved) to keep the kernel inside 256 registers.
+// K fragment of k-step ks, key block kvb: lane reads key row pi(lane%32) (+32 for the second block), chunk 2ks + lane/32
 template <int HD>
-struct QSplit {
-    static constexpr int KS = HD / 16;
-    static constexpr int QREG = KS;     // all of Q fits since the step exists in a single copy
-    static constexpr int QLDS = KS - QREG;
-};
+__device__ __forceinline__ bf16x8 k_frag(const char* sk, int ks, int kvb, int lane) {
+    return *reinterpret_cast<const bf16x8*>(sk + (lane >> 5) * 1024 + key_perm(lane & 31) * 16 + ks * 2048 + kvb * 512);
+}
+// V^T fragment of key chunk pair j (keys 16j..16j+15), channel block t: lane reads channel row 32t + lane%32, chunk 2j + lane/32
+template <int HD>
+__device__ __forceinline__ bf16x8 v_frag(const char* sv, int j, int t, int lane) {
+    return *reinterpret_cast<const bf16x8*>(sv + (lane >> 5) * (HD * 16) + (lane & 31) * 16 + j * (HD * 32) + t * 512);
+}
+
+// Whole score tile with plain just-in-time fragment reads (prologue only).
+template <int HD>
+__device__ __forceinline__ void scores_tile(const char* sk, const bf16x8 (&qf)[HD / 16], f32x16 (&s)[2], int lane) {
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks)
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+            s[kvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag<HD>(sk, ks, kvb, lane), qf[ks], s[kvb], 0, 0, 0);
+}
+
+constexpr int KWIN = 4;     // k-steps of K fragments kept in flight (x2 key blocks)
+constexpr int VWIN = 8;     // V^T fragments kept in flight
 
 template <int HD>
-__device__ __forceinline__ void scores_tile(const char* sk, const bf16x8 (&qf)[QSplit<HD>::QREG], const char* qstash,
-                                            f32x16 (&s)[2], int lane) {
-    // s holds the accumulator start values (-reference, or -inf for keys beyond the sequence end)
-    constexpr int QREG = QSplit<HD>::QREG;
-    // lane reads key row pi(lane%32) (+32 for the second block), chunk 2ks + lane/32
-    const char* base = sk + (lane >> 5) * 1024 + key_perm(lane & 31) * 16;
+__device__ __forceinline__ void preload_k(const char* sk, bf16x8 (&kw)[KWIN][2], int lane) {
 #pragma unroll
-    for (int ks = 0; ks < HD / 16; ++ks) {
-        bf16x8 q;
-        if (ks < QREG) q = qf[ks];
-        else q = *reinterpret_cast<const bf16x8*>(qstash + (ks - QREG) * 1024);
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + ks * 2048 + kvb * 512);
-            s[kvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q, s[kvb], 0, 0, 0);
-        }
+    for (int ks = 0; ks < KWIN; ++ks) {
+        kw[ks][0] = k_frag<HD>(sk, ks, 0, lane);
+        kw[ks][1] = k_frag<HD>(sk, ks, 1, lane);
     }
 }
 
-// Accumulator start values of a score tile: `start` everywhere, or -inf for keys >= keys_valid (ragged last
-// tile).  Register v of block kvb holds key 32 kvb + 16 (v/8) + 8 (lane/32) + v%8: the compile-time part is
-// compared against ONE per-lane threshold so that no per-register key index is ever materialised.
-__device__ __forceinline__ void init_scores(f32x16 (&s)[2], float start, bool ragged, int keys_valid, int lane) {
-    if (ragged) {      // wave-uniform
-        const int thr = keys_valid - 8 * (lane >> 5);
+// Scores of keys >= keys_valid (ragged last tile) become -inf.  Register v of block kvb holds key
+// 32 kvb + 16 (v/8) + 8 (lane/32) + v%8: the compile-time part is compared against ONE per-lane threshold so that
+// no per-register key index is ever materialised.
+__device__ __forceinline__ void mask_scores(f32x16 (&s)[2], int keys_valid, int lane) {
+    const int thr = keys_valid - 8 * (lane >> 5);
 #pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
+    for (int kvb = 0; kvb < 2; ++kvb)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int kc = 32 * kvb + 16 * (v >> 3) + (v & 7);
-                s[kvb][v] = (kc >= thr) ? -INFINITY : start;
-            }
-    } else {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) { s[0][v] = start; s[1][v] = start; }
-    }
+        for (int v = 0; v < 16; ++v) {
+            const int kc = 32 * kvb + 16 * (v >> 3) + (v & 7);
+            s[kvb][v] = (kc >= thr) ? -INFINITY : s[kvb][v];
+        }
 }
 
 __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
@@ -349,37 +348,34 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
     return __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
 }
 
-// One pipeline step.  s_cur (scores of tile j, accumulated on top of -m_ref) and mx_cur (its row maximum,
-// already reduced over the wave halves) come from the previous step.
-//   top      : rare branch - if a row maximum exceeds the reference by more than 2^kGrowLog2, move the reference
-//   block A  : S(j+1) MFMAs  ||  exp2 / bf16 pack / row-sum of tile j           (VALU under MFMA)
-//   block B  : O^T += V^T P^T MFMAs  ||  row maximum of S(j+1) for the next step
+// One pipeline step.  Everything the first MFMAs need is already in registers when the workgroup barrier at
+// the top of the step releases the wave, and all softmax arithmetic is placed under MFMAs:
+//   block A  : S(j+1) = K(j+1) Q^T, 16 MFMAs starting from literal zero (rolling K fragment window, first
+//              KWIN k-steps preloaded in the previous step)
+//              ||  p = exp2(s_cur - m_ref), bf16 pack, row sum of tile j ; first V^T fragments of tile j
+//   block B  : O^T += V^T P^T, 16 MFMAs (rolling V^T window)
+//              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
+//   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
+//              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
 template <int HD>
-__device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cur,
-                                          const bf16x8 (&qf)[QSplit<HD>::QREG], const char* qstash,
+__device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cur, const char* sk_next2,
+                                          const bf16x8 (&qf)[HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[2], f32x16 (&s_next)[2], f32x16 (&oacc)[HD / 32],
-                                          float& m_ref, float& mx_cur, float& l_run, int lane, bool next_ragged,
+                                          float& m_ref, float& l_run, int lane, bool next_ragged,
                                           int next_keys_valid) {
-    if (__builtin_amdgcn_ballot_w64(mx_cur > kGrowLog2) != 0) {
-        const float delta = mx_cur > kGrowLog2 ? mx_cur : 0.0f;
-        const float fac = __builtin_amdgcn_exp2f(-delta);
-        m_ref += delta;
-        l_run *= fac;
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s_cur[kvb][v] -= delta;
-#pragma unroll
-        for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[t][v] *= fac;
-    }
-    init_scores(s_next, -m_ref, next_ragged, next_keys_valid, lane);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K buffer and
+    constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
+    // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot and
     // their result is never used - cheaper than a second copy of the step.)
-    scores_tile<HD>(sk_next, qf, qstash, s_next, lane);
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        s_next[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][0], qf[ks], ks == 0 ? zero : s_next[0], 0, 0, 0);
+        s_next[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][1], qf[ks], ks == 0 ? zero : s_next[1], 0, 0, 0);
+        if (ks + KWIN < KS) {
+            kw[ks % KWIN][0] = k_frag<HD>(sk_next, ks + KWIN, 0, lane);
+            kw[ks % KWIN][1] = k_frag<HD>(sk_next, ks + KWIN, 1, lane);
+        }
+    }
     bf16x8 pf[4];
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
     float psum = 0.0f;
@@ -389,8 +385,8 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
 #pragma unroll
         for (int e = 0; e < 8; e += 2) {
             bf16x2 pp;
-            pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e]);
-            pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e + 1]);
+            pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e] - m_ref);
+            pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e + 1] - m_ref);
             psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
             p8[e] = pp[0];
             p8[e + 1] = pp[1];
@@ -398,39 +394,49 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
         pf[j] = p8;
     }
     l_run += psum;
-    // 16 MFMAs, 16 + QLDS fragment reads, ~64 VALU: a few reads up front, then per MFMA one or two reads and
-    // four VALU instructions
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+    bf16x8 vw[VWIN];
 #pragma unroll
-    for (int i = 0; i < QSplit<HD>::QLDS; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-    }
+    for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
+    // 2*KS MFMAs, 2*(KS-KWIN) + VWIN fragment reads, ~100 VALU: per MFMA one read and six VALU instructions
 #pragma unroll
-    for (int i = QSplit<HD>::QLDS; i < 2 * (HD / 16); ++i) {
+    for (int i = 0; i < 2 * KS; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
     }
+    // the probabilities must be complete here: without this the compiler sinks the whole exp/pack sequence past
+    // the branch below into block B, where it no longer fits under the MFMAs
+    asm volatile("" : "+v"(pf[0]), "+v"(pf[1]), "+v"(pf[2]), "+v"(pf[3]), "+v"(l_run));
     __builtin_amdgcn_sched_barrier(0);
+    if (next_ragged) mask_scores(s_next, next_keys_valid, lane);     // wave-uniform; only before a ragged last tile
 
-    // ---- block B: lane reads channel row 32t + lane%32, key chunk 2j + lane/32
-    const char* vb = sv_cur + (lane >> 5) * (HD * 16) + (lane & 31) * 16;
+    // ---- block B
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < NV; ++i) {
+        const int j = i / TS, t = i % TS;
+        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vw[i % VWIN], pf[j], oacc[t], 0, 0, 0);
+        if (i + VWIN < NV) vw[i % VWIN] = v_frag<HD>(sv_cur, (i + VWIN) / TS, (i + VWIN) % TS, lane);
+    }
+    const float mx = tile_row_max(s_next);
+    preload_k<HD>(sk_next2, kw, lane);
 #pragma unroll
-        for (int t = 0; t < HD / 32; ++t) {
-            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vb + j * (HD * 32) + t * 512);
-            oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[j], oacc[t], 0, 0, 0);
-        }
-    mx_cur = tile_row_max(s_next);
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-    for (int i = 0; i < 4 * (HD / 32); ++i) {
+    for (int i = 0; i < NV; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- tail
+    if (__builtin_amdgcn_ballot_w64(mx > m_ref + kGrowLog2) != 0) {
+        const float m_new = mx > m_ref + kGrowLog2 ? mx : m_ref;
+        const float fac = __builtin_amdgcn_exp2f(m_ref - m_new);
+        m_ref = m_new;
+        l_run *= fac;
+#pragma unroll
+        for (int t = 0; t < TS; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[t][v] *= fac;
     }
 }
 
@@ -460,9 +466,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int q0 = blockIdx.x * BMQ + wave * 32;
 
     // ---- Q fragments, pre-multiplied by log2(e)/sqrt(HD) (one extra bf16 rounding of Q)
-    constexpr int QREG = QSplit<HD>::QREG;
-    const char* qstash = nullptr;
-    bf16x8 qf[QREG];
+    bf16x8 qf[HD / 16];
     {
         int qrow = q0 + r32;
         qrow = qrow < p.n_tokens ? qrow : p.n_tokens - 1;
@@ -508,33 +512,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     issue(vbase, sv_addr, 0, 0);
     issue(kbase, sk_addr, 2, 2);
     issue(vbase, sv_addr, 1, 1);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * PER_WAVE) : "memory");   // K(0) has landed
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
     f32x16 s_a[2], s_b[2];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
-    init_scores(s_a, 0.0f, NT == 1 && ragged, last_valid, lane);
-    scores_tile<HD>(sk, qf, qstash, s_a, lane);
-    m_ref = tile_row_max(s_a);
-    float mx_cur = 0.0f;        // row maximum of the current scores relative to m_ref
 #pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s_a[kvb][v] -= m_ref;
+    for (int v = 0; v < 16; ++v) { s_a[0][v] = 0.0f; s_a[1][v] = 0.0f; }
+    scores_tile<HD>(sk, qf, s_a, lane);
+    if (NT == 1 && ragged) mask_scores(s_a, last_valid, lane);
+    m_ref = tile_row_max(s_a);      // exact first reference: every row has at least one finite score
+    bf16x8 kw[KWIN][2];
+    preload_k<HD>(sk + TILE_BYTES, kw, lane);      // K(1) for step 0
 
-    // step j: S(j+1) from K slot (j+1)%3, P(j) V(j) from V slot j%3; the loads of K(j+2), V(j+1) (issued one
-    // step ago) may still be in flight, those of K(j+1), V(j) (two steps ago) must have landed:
-    // s_waitcnt vmcnt(2 tiles).  After the barrier every wave is done with K(j) and V(j-1), whose slots are
-    // refilled with K(j+3) and V(j+2).
+    // step j: S(j+1) from K slot (j+1)%3, P(j) V(j) from V slot j%3, K(j+2) fragments preloaded from slot (j+2)%3.
+    // At the barrier everything but the most recently issued group, V(j+1), must have landed
+    // (s_waitcnt vmcnt(1 tile)): K(j+2) is read at the end of this very step.  After the barrier every wave is
+    // done with K(j) and V(j-1), whose slots are refilled with K(j+3) and V(j+2).
     int ks_next = 1, vs_cur = 0;      // ring slots: (j+1)%3 and j%3
 #define CDM_ATTN_STEP(SCUR, SNEXT)                                                                              \
     {                                                                                                           \
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER_WAVE) : "memory");                       \
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory");                           \
         const int k_fill = vs_cur;                              /* slot of K(j)   == j % 3     */               \
         const int v_fill = ks_next == 2 ? 0 : ks_next + 1;      /* slot of V(j-1) == (j+2) % 3 */               \
         issue(kbase, sk_addr, j + 3, k_fill);                                                                   \
         issue(vbase, sv_addr, j + 2, v_fill);                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
-        pipe_step<HD>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, qf, qstash, SCUR, SNEXT, oacc, m_ref,  \
-                      mx_cur, l_run, lane, ragged && j + 2 == NT, last_valid);                                  \
+        pipe_step<HD>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw, SCUR,  \
+                      SNEXT, oacc, m_ref, l_run, lane, ragged && j + 2 == NT, last_valid);              \
         vs_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }

@@ -36,7 +36,6 @@ struct GemmParams {
     const float* cos; const float* sin;
     int rope_cols, head_dim;
     int tiles_m, tiles_n;
-    int k_rotate;        // 1: each tile starts its K walk at its own offset
 };
 
 // chunk swizzle: 16-byte chunk c of tile row r lives at chunk position c ^ swz(r)
@@ -304,51 +303,51 @@ __device__ __forceinline__ bf16x8 lds_frag4(const char* tile, int row, int chunk
     return *reinterpret_cast<const bf16x8*>(tile + row * 64 + ((chunk ^ swz4(row)) << 4));
 }
 
-template <bool FP8>
-__device__ __forceinline__ void compute_stage4(const char* sa, const char* sb, f32x16 (&acc)[4][4], int wm, int wn,
-                                               int lane) {
+// fragments of one 16-element (bf16) / 64-element (e4m3, two chunks) k-step of a stage: 4 A + 4 W
+struct Frags {
+    bf16x8 a[4], b[4];
+};
+
+// k-step `ks` (0 or 1) of the stage at `sa`/`sb`.  bf16: chunk 2ks + kh.  e4m3: the stage is ONE 64-element MFMA
+// step whose operand is the chunk pair (2kh, 2kh+1); "ks" then selects the low or the high chunk of the pair.
+__device__ __forceinline__ void load_frags(Frags& f, const char* sa, const char* sb, int ks, int wm, int wn, int lane,
+                                           bool fp8) {
     const int r32 = lane & 31, kh = lane >> 5;
-    if (!FP8) {
+    const int chunk = fp8 ? 2 * kh + ks : 2 * ks + kh;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {     // 2 x 16 bf16 = 64 bytes
-            bf16x8 af[4], bfr[4];
+    for (int mi = 0; mi < 4; ++mi) f.a[mi] = lds_frag4(sa, wm * 128 + mi * 32 + r32, chunk);
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) af[mi] = lds_frag4(sa, wm * 128 + mi * 32 + r32, 2 * ks + kh);
+    for (int ni = 0; ni < 4; ++ni) f.b[ni] = lds_frag4(sb, wn * 128 + ni * 32 + r32, chunk);
+}
+
+__device__ __forceinline__ void mma_bf16(const Frags& f, f32x16 (&acc)[4][4]) {
 #pragma unroll
-            for (int ni = 0; ni < 4; ++ni) bfr[ni] = lds_frag4(sb, wn * 128 + ni * 32 + r32, 2 * ks + kh);
+    for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
+        for (int ni = 0; ni < 4; ++ni)
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[mi], f.b[ni], acc[mi][ni], 0, 0, 0);
+}
+
+__device__ __forceinline__ void mma_fp8(const Frags& lo, const Frags& hi, f32x16 (&acc)[4][4], int mi_begin,
+                                        int mi_end) {
 #pragma unroll
-                for (int ni = 0; ni < 4; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0);
-        }
-    } else {
-        i32x8 af[4], bfr[4];                 // 64 e4m3: one 32x32x64 MFMA step
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-            const int4 l4 = __builtin_bit_cast(int4, lds_frag4(sa, wm * 128 + mi * 32 + r32, 2 * kh));
-            const int4 h4 = __builtin_bit_cast(int4, lds_frag4(sa, wm * 128 + mi * 32 + r32, 2 * kh + 1));
-            af[mi] = i32x8{l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
-        }
+    for (int mi = 0; mi < 4; ++mi) {
+        if (mi < mi_begin || mi >= mi_end) continue;
+        const int4 al = __builtin_bit_cast(int4, lo.a[mi]), ah = __builtin_bit_cast(int4, hi.a[mi]);
+        const i32x8 av = {al.x, al.y, al.z, al.w, ah.x, ah.y, ah.z, ah.w};
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni) {
-            const int4 l4 = __builtin_bit_cast(int4, lds_frag4(sb, wn * 128 + ni * 32 + r32, 2 * kh));
-            const int4 h4 = __builtin_bit_cast(int4, lds_frag4(sb, wn * 128 + ni * 32 + r32, 2 * kh + 1));
-            bfr[ni] = i32x8{l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
+            const int4 bl = __builtin_bit_cast(int4, lo.b[ni]), bh = __builtin_bit_cast(int4, hi.b[ni]);
+            const i32x8 bv = {bl.x, bl.y, bl.z, bl.w, bh.x, bh.y, bh.z, bh.w};
+            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                          0x7f7f7f7f);
         }
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 4; ++ni)
-                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0,
-                                                                              0x7f7f7f7f, 0, 0x7f7f7f7f);
     }
 }
 
 __device__ __forceinline__ void issue_loads4(const char* abase, const char* wbase, const char* w2base,
                                              const uint32_t (&oa)[4], const uint32_t (&ob)[4], uint32_t w2mask,
-                                             char* sa, char* sb, int wave) {
-    const uint32_t la = lds_addr_of(sa) + wave * 1024, lb = lds_addr_of(sb) + wave * 1024;
+                                             uint32_t la, uint32_t lb) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         lds_dma16(abase, oa[i], la + i * 4096);
@@ -357,16 +356,18 @@ __device__ __forceinline__ void issue_loads4(const char* abase, const char* wbas
     }
 }
 
+// Schedule of one stage T (ring slot T & 3), with the fragments X of its first k-step already in registers:
+//     Y <- fragments of the second k-step                       (LDS reads fly under the next MFMAs)
+//     16 MFMAs on X
+//     wait: own Y reads done (this wave no longer needs slot T), tile T+1 landed; workgroup barrier
+//     refill slot T with tile T+4; X <- first k-step of tile T+1  (LDS reads fly under the next MFMAs)
+//     16 MFMAs on Y
+// so the matrix pipe always has queued work while LDS and global latencies are being paid, and the barrier
+// sits in the middle of a stage instead of in front of a fragment-read bubble.
 template <int EPI, bool FP8>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel4(const GemmParams p) {
-    __shared__ __attribute__((aligned(1024))) char sa0[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sb0[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sa1[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sb1[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sa2[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sb2[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sa3[kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char sb3[kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char s_a[4 * kStageBytes4];
+    __shared__ __attribute__((aligned(1024))) char s_b[4 * kStageBytes4];
 
     const int total = p.tiles_m * p.tiles_n;
     const int per_xcd = (total + 7) >> 3;
@@ -410,6 +411,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
     const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)n0 * p.ldw;
     const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)n0 * p.ldw : wbase;
+    const uint32_t la = lds_addr_of(s_a) + wave * 1024, lb = lds_addr_of(s_b) + wave * 1024;
 
     f32x16 acc[4][4];
 #pragma unroll
@@ -420,36 +422,34 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
             for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
     const int KT = p.K / (FP8 ? 64 : 32);   // k-tiles of 64 bytes; a multiple of 4 (host-checked)
-    // Every tile walks K from its own starting point (the sum over k is order-free).  With power-of-two row
-    // strides all 256 rows of a k-tile sit at the same offset modulo the stride, so workgroups marching
-    // through K in lockstep would all hit the same L2 / memory channels at the same time.
-    const int rot = p.k_rotate ? ((logical * 10) % KT) & ~1 : 0;
-    auto koff = [&](int t) {          // byte offset of the t-th k-tile this workgroup processes
-        int kk = t + rot;
-        kk = kk >= KT ? kk - KT : kk;
-        return kk * 64;
+    // tile index clamped to the last one: every stage issues the same 8 loads per wave, which keeps the
+    // s_waitcnt vmcnt(16) below valid up to the end (the surplus loads rewrite a free slot with the last tile)
+    auto issue = [&](int t, int slot) {
+        const int ko = (t < KT ? t : KT - 1) * 64;
+        issue_loads4(abase + ko, wbase + ko, w2base + ko, oa, ob, w2mask, la + slot * kStageBytes4,
+                     lb + slot * kStageBytes4);
     };
-    issue_loads4(abase + koff(0), wbase + koff(0), w2base + koff(0), oa, ob, w2mask, sa0, sb0, wave);
-    issue_loads4(abase + koff(1), wbase + koff(1), w2base + koff(1), oa, ob, w2mask, sa1, sb1, wave);
-    issue_loads4(abase + koff(2), wbase + koff(2), w2base + koff(2), oa, ob, w2mask, sa2, sb2, wave);
-    // stage t: wait for tile t (younger tiles stay in flight), barrier, refill the buffer freed by tile t-1
-#define CDM_STAGE(T, SA, SB, SA_FILL, SB_FILL)                                                              \
-    if ((T) + 2 < KT) asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");                        \
-    else if ((T) + 1 < KT) asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");                    \
-    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");                                      \
-    if ((T) + 3 < KT) {                                                                                     \
-        const int ko = koff((T) + 3);                                                                       \
-        issue_loads4(abase + ko, wbase + ko, w2base + ko, oa, ob, w2mask, SA_FILL, SB_FILL, wave);          \
-    }                                                                                                       \
-    __builtin_amdgcn_sched_barrier(0);                                                                      \
-    compute_stage4<FP8>(SA, SB, acc, wm, wn, lane);
+    issue(0, 0); issue(1, 1); issue(2, 2); issue(3, 3);
+    asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");     // tile 0 has landed everywhere
+    Frags X, Y;
+    load_frags(X, s_a, s_b, 0, wm, wn, lane, FP8);
+
+#define CDM_STAGE(T, SLOT, NEXT)                                                                                  \
+    load_frags(Y, s_a + (SLOT) * kStageBytes4, s_b + (SLOT) * kStageBytes4, 1, wm, wn, lane, FP8);                \
+    if (!FP8) mma_bf16(X, acc);                                                                                   \
+    else { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); mma_fp8(X, Y, acc, 0, 2); }                         \
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                     \
+    if (!FP8) { issue((T) + 4, SLOT); } else { mma_fp8(X, Y, acc, 2, 4); issue((T) + 4, SLOT); }                  \
+    load_frags(X, s_a + (NEXT) * kStageBytes4, s_b + (NEXT) * kStageBytes4, 0, wm, wn, lane, FP8);                \
+    if (!FP8) mma_bf16(Y, acc);
     for (int kt = 0; kt < KT; kt += 4) {
-        CDM_STAGE(kt, sa0, sb0, sa3, sb3)
-        CDM_STAGE(kt + 1, sa1, sb1, sa0, sb0)
-        CDM_STAGE(kt + 2, sa2, sb2, sa1, sb1)
-        CDM_STAGE(kt + 3, sa3, sb3, sa2, sb2)
+        CDM_STAGE(kt, 0, 1)
+        CDM_STAGE(kt + 1, 1, 2)
+        CDM_STAGE(kt + 2, 2, 3)
+        CDM_STAGE(kt + 3, 3, 0)
     }
 #undef CDM_STAGE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // surplus loads must not outlive the workgroup's LDS
     epilogue<EPI, FP8>(p, acc, m0, n0, wm, wn, lane);
 }
 
@@ -493,10 +493,7 @@ int32_t run(GemmParams& p, int64_t M, int64_t N, int32_t epilogue, hipStream_t s
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    // variant 0 = four-stage pipeline with per-tile K rotation (default); 1 = two-stage; 2 = four-stage, no rotation
-    const int variant = cdm_get_variant(1);
-    const bool deep = variant != 1;
-    p.k_rotate = variant == 0;
+    const bool deep = cdm_get_variant(1) != 1;     // variant 0 = four-slot ring pipeline (default), 1 = two-stage
 #define CDM_LAUNCH(E)                                                         \
     if (deep) gemm_kernel4<E, FP8><<<grid, kThreads, 0, st>>>(p);             \
     else gemm_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p)
