@@ -67,6 +67,7 @@ def main():
     ap.add_argument("--blocks", type=int, default=0, help="override the number of blocks (measurement aid; 0 = config)")
     ap.add_argument("--attn-variant", type=int, default=0)
     ap.add_argument("--gemm-variant", type=int, default=0)
+    ap.add_argument("--rope", default="in_attention", choices=["in_attention", "gemm_epilogue", "streaming"])
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -91,6 +92,10 @@ def main():
 
     stack = DMStack(cfg, device=dev)
     stack.reset_parameters()
+    if args.rope != "in_attention":
+        from cosmos_amd import DMAttnProcessor
+        for blk in stack.blocks:
+            blk.attn.set_processor(DMAttnProcessor(rope=args.rope))
     g = torch.Generator(device=dev).manual_seed(cfg.seed)
     xv = torch.randn((1, cfg.n_video, cfg.d_model), generator=g, device=dev).to(torch.bfloat16)
     xt = torch.randn((1, cfg.n_text, cfg.d_model), generator=g, device=dev).to(torch.bfloat16) if cfg.n_text else None
@@ -130,7 +135,7 @@ def main():
         "config": {"workload": f"{cfg.name}: {cfg.n_blocks} DM blocks, d={cfg.d_model}, {cfg.n_heads}x{cfg.head_dim} heads, "
                                f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
-                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant},
+                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4), "traffic": None,
                      "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},

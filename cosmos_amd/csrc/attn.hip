@@ -1,17 +1,16 @@
 // Non-causal full self-attention (flash-style, online softmax) on the gfx950 matrix cores.
 //
 // Work split: one workgroup owns 256 query rows of one head and streams all keys in tiles of 64.
-// Each wave owns 32*QSUB query rows.  Scores are computed TRANSPOSED, S^T = K . Q^T, with
-// v_mfma_f32_32x32x16_bf16: the A operand is a K tile row (plain 16-byte LDS read), the B operand
-// is Q held in registers for the whole kernel.  In the accumulator layout every lane then owns ONE
-// query column and 16 keys per 32-key block, so the row max / row sum of the online softmax are
-// in-lane reductions plus one exchange between the two half-waves.  The probabilities never move
-// between lanes: packed to bf16 they are already the B operand of O^T += V^T . P^T, whose A operand
-// is a row of V^T (V is transposed once per call into the caller's workspace, [head][dh][token]).
-// The K rows of a 32-key block are fetched in a permuted order so that the 8 keys a lane holds in
-// accumulator registers 8j..8j+7 are the 8 consecutive keys the second product expects.
-// K and V^T tiles go global -> LDS directly (global_load_lds_dwordx4), double buffered, with an
-// XOR swizzle applied on the source side so fragment reads are bank-conflict free.
+// Scores are computed TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_32x32x16_bf16: the A operand is a K
+// tile row (plain 16-byte LDS read), the B operand is Q held in registers for the whole kernel.  In
+// the accumulator layout every lane then owns ONE query column and 16 keys per 32-key block, so the
+// row max / row sum of the online softmax are in-lane reductions plus one exchange between the two
+// half-waves.  The probabilities never move between lanes: packed to bf16 they are already the B
+// operand of O^T += V^T . P^T, whose A operand is a row of V^T.  The K rows of a 32-key block are
+// fetched in a permuted order so that the 8 keys a lane holds in accumulator registers 8j..8j+7 are
+// the 8 consecutive keys the second product expects.
+// Rotate-half mRoPE is applied in registers: to K while it is re-tiled for the kernel, to Q when the
+// kernel loads its Q fragments (both members of a rotary pair sit in the same lane).
 #include "cdm_common.h"
 
 namespace {
@@ -20,263 +19,14 @@ constexpr int BN = 64;       // keys per tile
 constexpr int BMQ = 256;     // query rows per workgroup
 typedef __attribute__((address_space(3))) void lds_void;
 
-template <int CHUNKS>
-__device__ __forceinline__ int swz(int row) {
-    return CHUNKS == 16 ? (row & 15) : ((row ^ (row >> 3)) & 7);
-}
-
 // row permutation inside a 32-key block: MFMA output row i holds key pi(i)
 __device__ __forceinline__ int key_perm(int i) {
     const int g = i >> 3, b = (i >> 2) & 1, r = i & 3;
     return 16 * (g >> 1) + 8 * b + 4 * (g & 1) + r;
 }
 
-struct AttnParams {
-    const bf16_t* q; int64_t ldq;
-    const bf16_t* k; int64_t ldk;
-    const bf16_t* vt;            // [n_heads][HD][n_pad]
-    bf16_t* o; int64_t ldo;
-    int n_tokens, n_pad, n_heads;
-    float scale_log2e;           // log2(e) / sqrt(HD)
-};
-
-template <int HD, int QSUB, int NW>
-struct Cfg {
-    static constexpr int KCH = HD / 8;                   // 16-byte chunks per K tile row
-    static constexpr int K_TILE_BYTES = BN * HD * 2;
-    static constexpr int V_TILE_BYTES = HD * BN * 2;
-    static constexpr int K_INSTR = K_TILE_BYTES / 1024;  // wave-level direct-to-LDS instructions per tile
-    static constexpr int V_INSTR = V_TILE_BYTES / 1024;
-    static constexpr int K_PER_WAVE = K_INSTR / NW;
-    static constexpr int V_PER_WAVE = V_INSTR / NW;
-    static constexpr int K_ROWS_PER_INSTR = 64 / KCH;    // 4 (HD=128) or 8 (HD=64)
-    static_assert(K_INSTR % NW == 0 && V_INSTR % NW == 0, "tile loads must divide over the waves");
-};
-
-template <int HD, int QSUB, int NW>
-__device__ __forceinline__ void issue_tile(const char* kbase, const char* vbase,
-                                           const uint32_t (&ko)[Cfg<HD, QSUB, NW>::K_PER_WAVE],
-                                           const uint32_t (&vo)[Cfg<HD, QSUB, NW>::V_PER_WAVE], char* sk, char* sv,
-                                           int wave) {
-    using C = Cfg<HD, QSUB, NW>;
-#pragma unroll
-    for (int i = 0; i < C::K_PER_WAVE; ++i)
-        __builtin_amdgcn_global_load_lds(kbase + ko[i], (lds_void*)(sk + (i * NW + wave) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < C::V_PER_WAVE; ++i)
-        __builtin_amdgcn_global_load_lds(vbase + vo[i], (lds_void*)(sv + (i * NW + wave) * 1024), 16, 0, 0);
-}
-
-template <int HD, int QSUB, int NW>
-__device__ __forceinline__ void k_offsets(int wave, int lane, int64_t ldk, int rows_valid,
-                                          uint32_t (&ko)[Cfg<HD, QSUB, NW>::K_PER_WAVE]) {
-    using C = Cfg<HD, QSUB, NW>;
-#pragma unroll
-    for (int i = 0; i < C::K_PER_WAVE; ++i) {
-        const int row = (i * NW + wave) * C::K_ROWS_PER_INSTR + lane / C::KCH;
-        const int chunk = (lane % C::KCH) ^ swz<C::KCH>(row);
-        const int rr = row < rows_valid ? row : rows_valid - 1;
-        ko[i] = (uint32_t)(rr * (int)ldk + chunk * 8) * 2u;
-    }
-}
-
-// One key tile: S^T = K Q^T, online softmax, O^T += V^T P^T.
-template <int HD, int QSUB, int NW>
-__device__ __forceinline__ void process_tile(const char* sk, const char* sv, const bf16x8 (&qf)[QSUB][HD / 16],
-                                             f32x16 (&oacc)[QSUB][HD / 32], float (&m_run)[QSUB],
-                                             float (&l_run)[QSUB], float c, int lane, int keys_valid) {
-    using C = Cfg<HD, QSUB, NW>;
-    const int r32 = lane & 31, kh = lane >> 5;
-    const int prow = key_perm(r32);
-
-    f32x16 s[QSUB][2];
-#pragma unroll
-    for (int qs = 0; qs < QSUB; ++qs)
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s[qs][kvb][v] = 0.0f;
-
-#pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb) {
-        const int row = kvb * 32 + prow;
-        const char* rowp = sk + row * (HD * 2);
-        const int sw = swz<C::KCH>(row);
-#pragma unroll
-        for (int ks = 0; ks < HD / 16; ++ks) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(rowp + (((2 * ks + kh) ^ sw) << 4));
-#pragma unroll
-            for (int qs = 0; qs < QSUB; ++qs)
-                s[qs][kvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qs][ks], s[qs][kvb], 0, 0, 0);
-        }
-    }
-
-    bf16x8 pf[QSUB][4];
-#pragma unroll
-    for (int qs = 0; qs < QSUB; ++qs) {
-        if (keys_valid < BN) {   // wave-uniform: only the last, ragged tile
-#pragma unroll
-            for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int key = 32 * kvb + 16 * (v >> 3) + 8 * kh + (v & 7);
-                    if (key >= keys_valid) s[qs][kvb][v] = -INFINITY;
-                }
-        }
-        float mx = s[qs][0][0];
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[qs][kvb][v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[qs], mx * c);
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qs] - m_new);
-        const bool grew = m_new > m_run[qs];
-        m_run[qs] = m_new;
-        float psum = 0.0f;
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float pv = __builtin_amdgcn_exp2f(s[qs][kvb][v] * c - m_new);
-                s[qs][kvb][v] = pv;
-                psum += pv;
-            }
-        l_run[qs] = l_run[qs] * alpha + psum;
-        if (__builtin_amdgcn_ballot_w64(grew) != 0) {    // rescale only when some row's max moved
-#pragma unroll
-            for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) oacc[qs][t][v] *= alpha;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            bf16x8 p8;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) p8[e] = (__bf16)s[qs][j >> 1][8 * (j & 1) + e];
-            pf[qs][j] = p8;
-        }
-    }
-
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int t = 0; t < HD / 32; ++t) {
-            const int row = 32 * t + r32;
-            const bf16x8 vf =
-                *reinterpret_cast<const bf16x8*>(sv + row * (BN * 2) + (((2 * j + kh) ^ swz<8>(row)) << 4));
-#pragma unroll
-            for (int qs = 0; qs < QSUB; ++qs)
-                oacc[qs][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qs][j], oacc[qs][t], 0, 0, 0);
-        }
-}
-
-template <int HD, int QSUB, int NW>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4))) void attn_fwd_kernel(
-    const AttnParams p) {
-    using C = Cfg<HD, QSUB, NW>;
-    static_assert(QSUB * NW * 32 == BMQ, "workgroup must cover BMQ query rows");
-    __shared__ __attribute__((aligned(1024))) char sk0[C::K_TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char sv0[C::V_TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char sk1[C::K_TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char sv1[C::V_TILE_BYTES];
-
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r32 = lane & 31, kh = lane >> 5;
-    const int qtile = blockIdx.x, head = blockIdx.y;
-    const int q0 = qtile * BMQ + wave * (32 * QSUB);
-
-    // ---- Q fragments (B operand of S^T = K Q^T): lane holds query r32, channels 16ks + 8kh .. +7
-    bf16x8 qf[QSUB][HD / 16];
-#pragma unroll
-    for (int qs = 0; qs < QSUB; ++qs) {
-        int qrow = q0 + qs * 32 + r32;
-        qrow = qrow < p.n_tokens ? qrow : p.n_tokens - 1;
-        const bf16_t* qp = p.q + (int64_t)qrow * p.ldq + head * HD + 8 * kh;
-#pragma unroll
-        for (int ks = 0; ks < HD / 16; ++ks) qf[qs][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
-    }
-
-    f32x16 oacc[QSUB][HD / 32];
-    float m_run[QSUB], l_run[QSUB];
-#pragma unroll
-    for (int qs = 0; qs < QSUB; ++qs) {
-        m_run[qs] = -INFINITY;
-        l_run[qs] = 0.0f;
-#pragma unroll
-        for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[qs][t][v] = 0.0f;
-    }
-
-    // ---- per-lane byte offsets of this wave's share of the tile loads
-    uint32_t ko[C::K_PER_WAVE], ko_last[C::K_PER_WAVE], vo[C::V_PER_WAVE];
-    const int NT = (p.n_tokens + BN - 1) / BN;
-    const int last_valid = p.n_tokens - (NT - 1) * BN;      // keys in the last tile (1..64)
-    k_offsets<HD, QSUB, NW>(wave, lane, p.ldk, BN, ko);
-    k_offsets<HD, QSUB, NW>(wave, lane, p.ldk, last_valid, ko_last);
-#pragma unroll
-    for (int i = 0; i < C::V_PER_WAVE; ++i) {
-        const int row = (i * NW + wave) * 8 + (lane >> 3);
-        const int chunk = (lane & 7) ^ swz<8>(row);
-        vo[i] = (uint32_t)(row * p.n_pad + chunk * 8) * 2u;
-    }
-    const char* kbase = reinterpret_cast<const char*>(p.k + head * HD);
-    const char* vbase = reinterpret_cast<const char*>(p.vt + (int64_t)head * HD * p.n_pad);
-    const int64_t kstep = (int64_t)BN * p.ldk * 2;    // bytes per key tile
-    const int64_t vstep = (int64_t)BN * 2;
-    const float c = p.scale_log2e;
-
-    // tile j lives in buffer j & 1
-    if (NT == 1) issue_tile<HD, QSUB, NW>(kbase, vbase, ko_last, vo, sk0, sv0, wave);
-    else issue_tile<HD, QSUB, NW>(kbase, vbase, ko, vo, sk0, sv0, wave);
-    int j = 0;
-    for (; j + 1 < NT; j += 2) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (j + 2 == NT) issue_tile<HD, QSUB, NW>(kbase + (j + 1) * kstep, vbase + (j + 1) * vstep, ko_last, vo, sk1, sv1, wave);
-        else issue_tile<HD, QSUB, NW>(kbase + (j + 1) * kstep, vbase + (j + 1) * vstep, ko, vo, sk1, sv1, wave);
-        __builtin_amdgcn_sched_barrier(0);
-        process_tile<HD, QSUB, NW>(sk0, sv0, qf, oacc, m_run, l_run, c, lane, BN);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (j + 2 < NT) {
-            if (j + 3 == NT) issue_tile<HD, QSUB, NW>(kbase + (j + 2) * kstep, vbase + (j + 2) * vstep, ko_last, vo, sk0, sv0, wave);
-            else issue_tile<HD, QSUB, NW>(kbase + (j + 2) * kstep, vbase + (j + 2) * vstep, ko, vo, sk0, sv0, wave);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        process_tile<HD, QSUB, NW>(sk1, sv1, qf, oacc, m_run, l_run, c, lane, (j + 2 == NT) ? last_valid : BN);
-    }
-    if (j < NT) {   // odd tile count: the last tile sits in buffer 0
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        process_tile<HD, QSUB, NW>(sk0, sv0, qf, oacc, m_run, l_run, c, lane, last_valid);
-    }
-
-    // ---- normalise and store: lane owns query r32; accumulator v of block t is channel 32t + 8(v/4) + 4kh + v%4
-#pragma unroll
-    for (int qs = 0; qs < QSUB; ++qs) {
-        const float l_tot = l_run[qs] + __shfl_xor(l_run[qs], 32, 64);
-        const float inv = 1.0f / l_tot;
-        const int qrow = q0 + qs * 32 + r32;
-        if (qrow < p.n_tokens) {
-            bf16_t* op = p.o + (int64_t)qrow * p.ldo + head * HD + 4 * kh;
-#pragma unroll
-            for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    uint2 w;
-                    w.x = pack_bf16x2(oacc[qs][t][4 * g + 0] * inv, oacc[qs][t][4 * g + 1] * inv);
-                    w.y = pack_bf16x2(oacc[qs][t][4 * g + 2] * inv, oacc[qs][t][4 * g + 3] * inv);
-                    *reinterpret_cast<uint2*>(op + 32 * t + 8 * g) = w;
-                }
-        }
-    }
-}
-
 // ---------------------------------------------------------------------------------------------
-// Software-pipelined kernel (8 waves x 32 query rows) over PRE-TILED K and V.
+// Software-pipelined kernel over PRE-TILED K and V.
 //  * K and V are first re-laid out in the workspace as the exact LDS image of each 64-key tile,
 //    chunk-major:  Kp[head][tile][c = dh/8][key r = 0..63][8 ch]   and
 //                  Vp[head][tile][c = key/8 (0..7)][channel row = 0..HD-1][8 keys]  (V transposed).
@@ -357,70 +107,87 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-template <int HD>
+template <int HD, int QS>
 __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cur, const char* sk_next2,
-                                          const bf16x8 (&qf)[HD / 16], bf16x8 (&kw)[KWIN][2],
-                                          f32x16 (&s_cur)[2], f32x16 (&s_next)[2], f32x16 (&oacc)[HD / 32],
-                                          float& m_ref, float& l_run, int lane, bool next_ragged,
-                                          int next_keys_valid) {
+                                          const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
+                                          f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
+                                          f32x16 (&oacc)[QS][HD / 32], float (&m_ref)[QS], float (&l_run)[QS], int lane,
+                                          bool next_ragged, int next_keys_valid) {
     constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
     // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot and
     // their result is never used - cheaper than a second copy of the step.)
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        s_next[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][0], qf[ks], ks == 0 ? zero : s_next[0], 0, 0, 0);
-        s_next[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][1], qf[ks], ks == 0 ? zero : s_next[1], 0, 0, 0);
+#pragma unroll
+        for (int qs = 0; qs < QS; ++qs) {
+            s_next[qs][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][0], qf[qs][ks],
+                                                                    ks == 0 ? zero : s_next[qs][0], 0, 0, 0);
+            s_next[qs][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][1], qf[qs][ks],
+                                                                    ks == 0 ? zero : s_next[qs][1], 0, 0, 0);
+        }
         if (ks + KWIN < KS) {
             kw[ks % KWIN][0] = k_frag<HD>(sk_next, ks + KWIN, 0, lane);
             kw[ks % KWIN][1] = k_frag<HD>(sk_next, ks + KWIN, 1, lane);
         }
     }
-    bf16x8 pf[4];
+    bf16x8 pf[QS][4];
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-    float psum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        bf16x8 p8;
+    for (int qs = 0; qs < QS; ++qs) {
+        float psum = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; e += 2) {
-            bf16x2 pp;
-            pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e] - m_ref);
-            pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[j >> 1][8 * (j & 1) + e + 1] - m_ref);
-            psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
-            p8[e] = pp[0];
-            p8[e + 1] = pp[1];
+        for (int j = 0; j < 4; ++j) {
+            bf16x8 p8;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                bf16x2 pp;
+                pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e] - m_ref[qs]);
+                pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1] - m_ref[qs]);
+                psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
+                p8[e] = pp[0];
+                p8[e + 1] = pp[1];
+            }
+            pf[qs][j] = p8;
         }
-        pf[j] = p8;
+        l_run[qs] += psum;
     }
-    l_run += psum;
     bf16x8 vw[VWIN];
 #pragma unroll
     for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
-    // 2*KS MFMAs, 2*(KS-KWIN) + VWIN fragment reads, ~100 VALU: per MFMA one read and six VALU instructions
+    // per MFMA (at most) one fragment read and six VALU instructions
 #pragma unroll
-    for (int i = 0; i < 2 * KS; ++i) {
+    for (int i = 0; i < 2 * KS * QS; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
     }
     // the probabilities must be complete here: without this the compiler sinks the whole exp/pack sequence past
     // the branch below into block B, where it no longer fits under the MFMAs
-    asm volatile("" : "+v"(pf[0]), "+v"(pf[1]), "+v"(pf[2]), "+v"(pf[3]), "+v"(l_run));
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs)
+        asm volatile("" : "+v"(pf[qs][0]), "+v"(pf[qs][1]), "+v"(pf[qs][2]), "+v"(pf[qs][3]), "+v"(l_run[qs]));
     __builtin_amdgcn_sched_barrier(0);
-    if (next_ragged) mask_scores(s_next, next_keys_valid, lane);     // wave-uniform; only before a ragged last tile
+    if (next_ragged) {     // wave-uniform; only before a ragged last tile
+#pragma unroll
+        for (int qs = 0; qs < QS; ++qs) mask_scores(s_next[qs], next_keys_valid, lane);
+    }
 
     // ---- block B
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int j = i / TS, t = i % TS;
-        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vw[i % VWIN], pf[j], oacc[t], 0, 0, 0);
+#pragma unroll
+        for (int qs = 0; qs < QS; ++qs)
+            oacc[qs][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vw[i % VWIN], pf[qs][j], oacc[qs][t], 0, 0, 0);
         if (i + VWIN < NV) vw[i % VWIN] = v_frag<HD>(sv_cur, (i + VWIN) / TS, (i + VWIN) % TS, lane);
     }
-    const float mx = tile_row_max(s_next);
+    float mx[QS];
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
     preload_k<HD>(sk_next2, kw, lane);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
+    for (int i = 0; i < NV * QS; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
@@ -428,15 +195,18 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- tail
-    if (__builtin_amdgcn_ballot_w64(mx > m_ref + kGrowLog2) != 0) {
-        const float m_new = mx > m_ref + kGrowLog2 ? mx : m_ref;
-        const float fac = __builtin_amdgcn_exp2f(m_ref - m_new);
-        m_ref = m_new;
-        l_run *= fac;
 #pragma unroll
-        for (int t = 0; t < TS; ++t)
+    for (int qs = 0; qs < QS; ++qs) {
+        if (__builtin_amdgcn_ballot_w64(mx[qs] > m_ref[qs] + kGrowLog2) != 0) {
+            const float m_new = mx[qs] > m_ref[qs] + kGrowLog2 ? mx[qs] : m_ref[qs];
+            const float fac = __builtin_amdgcn_exp2f(m_ref[qs] - m_new);
+            m_ref[qs] = m_new;
+            l_run[qs] *= fac;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[t][v] *= fac;
+            for (int t = 0; t < TS; ++t)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) oacc[qs][t][v] *= fac;
+        }
     }
 }
 
@@ -445,14 +215,18 @@ struct PackedParams {
     const char* kp;              // [n_heads][n_tiles][tile bytes]
     const char* vp;
     bf16_t* o; int64_t ldo;
+    const float* cos; const float* sin;   // optional rotary tables [n_tokens, HD/2] applied to Q at load
     int n_tokens, n_heads;
     float scale_log2e;
 };
 
-template <int HD>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_pipe_kernel(
+// QS = query sub-tiles (of 32 rows) per wave: QS = 1 -> 8 waves, two per SIMD, 256 registers each;
+// QS = 2 -> 4 waves, one per SIMD with the 512-register budget; every K / V^T fragment read from LDS then feeds
+// two MFMAs instead of one.
+template <int HD, int QS>
+__global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS, 2 / QS))) void attn_fwd_pipe_kernel(
     const PackedParams p) {
-    constexpr int NW = 8;
+    constexpr int NW = 8 / QS;
     constexpr int TILE_BYTES = BN * HD * 2;            // same for K and V tiles
     constexpr int PER_WAVE = TILE_BYTES / 1024 / NW;   // direct-to-LDS instructions per wave per tile
     constexpr int RING = 3;                            // K(t) lives in slot t % 3, V(t) in slot t % 3
@@ -463,32 +237,62 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r32 = lane & 31, kh = lane >> 5;
     const int head = blockIdx.y;
-    const int q0 = blockIdx.x * BMQ + wave * 32;
+    const int q0 = blockIdx.x * BMQ + wave * (32 * QS);
 
-    // ---- Q fragments, pre-multiplied by log2(e)/sqrt(HD) (one extra bf16 rounding of Q)
-    bf16x8 qf[HD / 16];
-    {
-        int qrow = q0 + r32;
+    // ---- Q fragments: rotate-half mRoPE (if tables are given) and the factor log2(e)/sqrt(HD), both in fp32 and
+    // with ONE rounding to bf16.  The lane holds channels 16ks + 8kh .. +7 of its query row for every ks, so
+    // the partner of a channel in k-step ks (< KS/2) is the same register element of k-step ks + KS/2.
+    bf16x8 qf[QS][HD / 16];
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs) {
+        constexpr int KS = HD / 16;
+        int qrow = q0 + qs * 32 + r32;
         qrow = qrow < p.n_tokens ? qrow : p.n_tokens - 1;
         const bf16_t* qp = p.q + (int64_t)qrow * p.ldq + head * HD + 8 * kh;
+        uint4 raw[KS];
 #pragma unroll
-        for (int ks = 0; ks < HD / 16; ++ks) {
-            const uint4 u = *reinterpret_cast<const uint4*>(qp + 16 * ks);
-            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
-            uint32_t o[4];
+        for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qp + 16 * ks);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16lo(w[e]) * p.scale_log2e, bf16hi(w[e]) * p.scale_log2e);
-            qf[ks] = __builtin_bit_cast(bf16x8, make_uint4(o[0], o[1], o[2], o[3]));
+        for (int ks = 0; ks < KS / 2; ++ks) {
+            const uint32_t w1[4] = {raw[ks].x, raw[ks].y, raw[ks].z, raw[ks].w};
+            const uint32_t w2[4] = {raw[ks + KS / 2].x, raw[ks + KS / 2].y, raw[ks + KS / 2].z, raw[ks + KS / 2].w};
+            float c[8], sn[8];
+            if (p.cos != nullptr) {
+                const float4* cp = reinterpret_cast<const float4*>(p.cos + (int64_t)qrow * (HD / 2) + 16 * ks + 8 * kh);
+                const float4* sp = reinterpret_cast<const float4*>(p.sin + (int64_t)qrow * (HD / 2) + 16 * ks + 8 * kh);
+                const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+                c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+                sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { c[e] = 1.0f; sn[e] = 0.0f; }
+            }
+            uint32_t o1[4], o2[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float a0 = bf16lo(w1[j]), a1 = bf16hi(w1[j]), b0 = bf16lo(w2[j]), b1 = bf16hi(w2[j]);
+                o1[j] = pack_bf16x2((a0 * c[2 * j] - b0 * sn[2 * j]) * p.scale_log2e,
+                                    (a1 * c[2 * j + 1] - b1 * sn[2 * j + 1]) * p.scale_log2e);
+                o2[j] = pack_bf16x2((b0 * c[2 * j] + a0 * sn[2 * j]) * p.scale_log2e,
+                                    (b1 * c[2 * j + 1] + a1 * sn[2 * j + 1]) * p.scale_log2e);
+            }
+            qf[qs][ks] = __builtin_bit_cast(bf16x8, make_uint4(o1[0], o1[1], o1[2], o1[3]));
+            qf[qs][ks + KS / 2] = __builtin_bit_cast(bf16x8, make_uint4(o2[0], o2[1], o2[2], o2[3]));
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // Q is in registers: from here on vmcnt counts tile loads only
 
-    f32x16 oacc[HD / 32];
+    f32x16 oacc[QS][HD / 32];
+    float m_ref[QS], l_run[QS];
 #pragma unroll
-    for (int t = 0; t < HD / 32; ++t)
+    for (int qs = 0; qs < QS; ++qs) {
+        m_ref[qs] = 0.0f;
+        l_run[qs] = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[t][v] = 0.0f;
-    float m_ref = 0.0f, l_run = 0.0f;
+        for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[qs][t][v] = 0.0f;
+    }
 
     const int NT = (p.n_tokens + BN - 1) / BN;
     const int last_valid = p.n_tokens - (NT - 1) * BN;
@@ -513,13 +317,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     issue(kbase, sk_addr, 2, 2);
     issue(vbase, sv_addr, 1, 1);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
-    f32x16 s_a[2], s_b[2];      // score tiles ping-pong between the two halves of the unrolled loop
+    f32x16 s_a[QS][2], s_b[QS][2];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) { s_a[0][v] = 0.0f; s_a[1][v] = 0.0f; }
-    scores_tile<HD>(sk, qf, s_a, lane);
-    if (NT == 1 && ragged) mask_scores(s_a, last_valid, lane);
-    m_ref = tile_row_max(s_a);      // exact first reference: every row has at least one finite score
+    for (int qs = 0; qs < QS; ++qs) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { s_a[qs][0][v] = 0.0f; s_a[qs][1][v] = 0.0f; }
+        scores_tile<HD>(sk, qf[qs], s_a[qs], lane);
+        if (NT == 1 && ragged) mask_scores(s_a[qs], last_valid, lane);
+        m_ref[qs] = tile_row_max(s_a[qs]);      // exact first reference: every row has at least one finite score
+    }
     bf16x8 kw[KWIN][2];
     preload_k<HD>(sk + TILE_BYTES, kw, lane);      // K(1) for step 0
 
@@ -536,8 +343,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         issue(kbase, sk_addr, j + 3, k_fill);                                                                   \
         issue(vbase, sv_addr, j + 2, v_fill);                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
-        pipe_step<HD>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw, SCUR,  \
-                      SNEXT, oacc, m_ref, l_run, lane, ragged && j + 2 == NT, last_valid);              \
+        pipe_step<HD, QS>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,  \
+                          SCUR, SNEXT, oacc, m_ref, l_run, lane, ragged && j + 2 == NT, last_valid);            \
         vs_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
@@ -549,46 +356,77 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #undef CDM_ATTN_STEP
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct-to-LDS write may outlive the workgroup
 
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / l_tot;
-    const int qrow = q0 + r32;
-    if (qrow < p.n_tokens) {
-        bf16_t* op = p.o + (int64_t)qrow * p.ldo + head * HD + 4 * kh;
 #pragma unroll
-        for (int t = 0; t < HD / 32; ++t)
+    for (int qs = 0; qs < QS; ++qs) {
+        const float l_tot = l_run[qs] + __shfl_xor(l_run[qs], 32, 64);
+        const float inv = 1.0f / l_tot;
+        const int qrow = q0 + qs * 32 + r32;
+        if (qrow < p.n_tokens) {
+            bf16_t* op = p.o + (int64_t)qrow * p.ldo + head * HD + 4 * kh;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint2 w;
-                w.x = pack_bf16x2(oacc[t][4 * g + 0] * inv, oacc[t][4 * g + 1] * inv);
-                w.y = pack_bf16x2(oacc[t][4 * g + 2] * inv, oacc[t][4 * g + 3] * inv);
-                *reinterpret_cast<uint2*>(op + 32 * t + 8 * g) = w;
-            }
+            for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    uint2 w;
+                    w.x = pack_bf16x2(oacc[qs][t][4 * g + 0] * inv, oacc[qs][t][4 * g + 1] * inv);
+                    w.y = pack_bf16x2(oacc[qs][t][4 * g + 2] * inv, oacc[qs][t][4 * g + 3] * inv);
+                    *reinterpret_cast<uint2*>(op + 32 * t + 8 * g) = w;
+                }
+        }
     }
 }
 
-// K, V [n_tokens, n_heads, HD] -> tile images Kp, Vp (see above); one workgroup per (64-key tile, head)
+// K, V [n_tokens, n_heads, HD] -> tile images Kp, Vp (see above); one workgroup per (64-key tile, head).
+// With cos/sin tables ([n_tokens, HD/2] fp32) K is rotated on the way (rotate-half pairs (i, i + HD/2)).
 template <int HD>
 __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__ k, int64_t ldk,
                                                       const bf16_t* __restrict__ v, int64_t ldv,
+                                                      const float* __restrict__ cos, const float* __restrict__ sin,
                                                       char* __restrict__ kp, char* __restrict__ vp, int n_tokens,
                                                       int n_tiles) {
     __shared__ bf16_t tile[64][HD + 2];
     constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
+    constexpr int HALF = HD / 2;
     constexpr int TILE_BYTES = BN * HD * 2;
     const int tile_idx = blockIdx.x, head = blockIdx.y;
     const int t0 = tile_idx * 64;
     char* kt = kp + ((int64_t)head * n_tiles + tile_idx) * TILE_BYTES;
     char* vt = vp + ((int64_t)head * n_tiles + tile_idx) * TILE_BYTES;
-    for (int idx = threadIdx.x; idx < 64 * CPR; idx += 256) {
-        const int r = idx / CPR, ch = idx % CPR;
-        uint4 uk = make_uint4(0, 0, 0, 0), uv = uk;
+    // one thread handles the chunk pair (ch, ch + CPR/2) of one token: the two halves of 8 rotary pairs
+    for (int idx = threadIdx.x; idx < 64 * (CPR / 2); idx += 256) {
+        const int r = idx / (CPR / 2), ch = idx % (CPR / 2);
+        uint4 k1 = make_uint4(0, 0, 0, 0), k2 = k1, v1 = k1, v2 = k1;
         if (t0 + r < n_tokens) {
-            uk = *reinterpret_cast<const uint4*>(k + (int64_t)(t0 + r) * ldk + head * HD + ch * 8);
-            uv = *reinterpret_cast<const uint4*>(v + (int64_t)(t0 + r) * ldv + head * HD + ch * 8);
+            const bf16_t* kr = k + (int64_t)(t0 + r) * ldk + head * HD + ch * 8;
+            const bf16_t* vr = v + (int64_t)(t0 + r) * ldv + head * HD + ch * 8;
+            k1 = *reinterpret_cast<const uint4*>(kr);
+            k2 = *reinterpret_cast<const uint4*>(kr + HALF);
+            v1 = *reinterpret_cast<const uint4*>(vr);
+            v2 = *reinterpret_cast<const uint4*>(vr + HALF);
+            if (cos != nullptr) {
+                const float4* cp = reinterpret_cast<const float4*>(cos + (int64_t)(t0 + r) * HALF + ch * 8);
+                const float4* sp = reinterpret_cast<const float4*>(sin + (int64_t)(t0 + r) * HALF + ch * 8);
+                const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+                const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+                const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+                const uint32_t w1[4] = {k1.x, k1.y, k1.z, k1.w}, w2[4] = {k2.x, k2.y, k2.z, k2.w};
+                uint32_t o1[4], o2[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float a0 = bf16lo(w1[j]), a1 = bf16hi(w1[j]), b0 = bf16lo(w2[j]), b1 = bf16hi(w2[j]);
+                    o1[j] = pack_bf16x2(a0 * c[2 * j] - b0 * sn[2 * j], a1 * c[2 * j + 1] - b1 * sn[2 * j + 1]);
+                    o2[j] = pack_bf16x2(b0 * c[2 * j] + a0 * sn[2 * j], b1 * c[2 * j + 1] + a1 * sn[2 * j + 1]);
+                }
+                k1 = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+                k2 = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+            }
         }
-        *reinterpret_cast<uint4*>(kt + (ch * 64 + r) * 16) = uk;          // chunk-major K image
-        uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[r][ch * 8]);
-        dst[0] = uv.x; dst[1] = uv.y; dst[2] = uv.z; dst[3] = uv.w;
+        *reinterpret_cast<uint4*>(kt + (ch * 64 + r) * 16) = k1;                  // chunk-major K image
+        *reinterpret_cast<uint4*>(kt + ((ch + CPR / 2) * 64 + r) * 16) = k2;
+        uint32_t* d1 = reinterpret_cast<uint32_t*>(&tile[r][ch * 8]);
+        uint32_t* d2 = reinterpret_cast<uint32_t*>(&tile[r][HALF + ch * 8]);
+        d1[0] = v1.x; d1[1] = v1.y; d1[2] = v1.z; d1[3] = v1.w;
+        d2[0] = v2.x; d2[1] = v2.y; d2[2] = v2.z; d2[3] = v2.w;
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < HD * 8; idx += 256) {
@@ -601,64 +439,34 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
     }
 }
 
-// V[n_tokens, n_heads, HD] (row stride ldv) -> Vt[n_heads][HD][n_pad], zero beyond n_tokens
-template <int HD>
-__global__ __launch_bounds__(256) void transpose_v_kernel(const bf16_t* __restrict__ v, int64_t ldv,
-                                                          bf16_t* __restrict__ vt, int n_tokens, int n_pad) {
-    __shared__ bf16_t tile[64][HD + 2];
-    const int t0 = blockIdx.x * 64, head = blockIdx.y;
-    constexpr int CPR = HD / 8;      // 16-byte chunks per token row
-    for (int idx = threadIdx.x; idx < 64 * CPR; idx += 256) {
-        const int r = idx / CPR, ch = idx % CPR;
-        uint4 u = make_uint4(0, 0, 0, 0);
-        if (t0 + r < n_tokens) u = *reinterpret_cast<const uint4*>(v + (int64_t)(t0 + r) * ldv + head * HD + ch * 8);
-        uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[r][ch * 8]);
-        dst[0] = u.x; dst[1] = u.y; dst[2] = u.z; dst[3] = u.w;
-    }
-    __syncthreads();
-    // each thread writes 8 consecutive tokens of one channel
-    for (int idx = threadIdx.x; idx < HD * 8; idx += 256) {
-        const int ch = idx >> 3, tg = idx & 7;
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            w[e] = (uint32_t)tile[tg * 8 + 2 * e][ch] | ((uint32_t)tile[tg * 8 + 2 * e + 1][ch] << 16);
-        *reinterpret_cast<uint4*>(vt + ((int64_t)head * HD + ch) * n_pad + t0 + tg * 8) = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-}
-
 inline int64_t pad_tokens(int64_t n) { return (n + BN - 1) / BN * BN; }
 inline int64_t image_bytes(int64_t n_tokens, int n_heads, int head_dim) {      // one packed tensor
     return pad_tokens(n_tokens) * n_heads * head_dim * 2;
 }
 
-template <int HD, int QSUB, int NW>
-void launch_attn(const AttnParams& p, hipStream_t st) {
-    dim3 grid((p.n_tokens + BMQ - 1) / BMQ, p.n_heads);
-    attn_fwd_kernel<HD, QSUB, NW><<<grid, NW * 64, 0, st>>>(p);
-}
-
-int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
+int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, int32_t head_dim, const float* cos,
+                          const float* sin) {
     CDM_REQUIRE(n_tokens >= 0 && n_heads > 0, CDM_ERR_BAD_ARG, "%s: bad sizes", who);
     CDM_REQUIRE(head_dim == 64 || head_dim == 128, CDM_ERR_BAD_SHAPE, "%s: head_dim=%d must be 64 or 128", who, head_dim);
     CDM_REQUIRE(n_tokens < (1ll << 23) && n_heads <= 65535, CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
+    CDM_REQUIRE((cos == nullptr) == (sin == nullptr), CDM_ERR_BAD_ARG, "%s: cos and sin must be given together", who);
+    CDM_REQUIRE(cdm_aligned16(cos) && cdm_aligned16(sin), CDM_ERR_BAD_ALIGN, "%s: rotary tables must be 16-byte aligned", who);
     return CDM_OK;
 }
 
 }  // namespace
 
-// workspace = [Kp | Vp | V^T]: the two tile images of the pipelined kernel, then the plain per-head
-// transpose of V that the non-pipelined variants read
+// workspace = [Kp | Vp]: the two tile images
 extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
     if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0) return 0;
-    return 3 * image_bytes(n_tokens, n_heads, head_dim);
+    return 2 * image_bytes(n_tokens, n_heads, head_dim);
 }
 
-extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, void* workspace,
-                                         int64_t workspace_bytes, int64_t n_tokens, int32_t n_heads,
-                                         int32_t head_dim, void* stream) {
+extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
+                                         const float* sin, void* workspace, int64_t workspace_bytes,
+                                         int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream) {
     CDM_REQUIRE(k && v && workspace, CDM_ERR_BAD_ARG, "attn_pack_kv: null pointer");
-    int32_t rc = check_attn_common("attn_pack_kv", n_tokens, n_heads, head_dim);
+    int32_t rc = check_attn_common("attn_pack_kv", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldk >= d && ldv >= d, CDM_ERR_BAD_ARG, "attn_pack_kv: row stride smaller than n_heads*head_dim");
@@ -675,18 +483,19 @@ extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void*
     dim3 grid(n_tiles, n_heads);
     hipStream_t st = (hipStream_t)stream;
     if (head_dim == 128)
-        pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, ws, ws + img,
+        pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, ws, ws + img,
                                                   (int)n_tokens, n_tiles);
     else
-        pack_kv_kernel<64><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, ws, ws + img,
+        pack_kv_kernel<64><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, ws, ws + img,
                                                  (int)n_tokens, n_tiles);
     return cdm_check_launch("attn_pack_kv");
 }
 
-extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const void* workspace, void* o, int64_t ldo,
-                                            int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream) {
+extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
+                                            const void* workspace, void* o, int64_t ldo, int64_t n_tokens,
+                                            int32_t n_heads, int32_t head_dim, void* stream) {
     CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
-    int32_t rc = check_attn_common("attn_fwd_packed", n_tokens, n_heads, head_dim);
+    int32_t rc = check_attn_common("attn_fwd_packed", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldq >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd_packed: row stride smaller than n_heads*head_dim");
@@ -699,61 +508,41 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const vo
     p.q = (const bf16_t*)q; p.ldq = ldq;
     p.kp = (const char*)workspace; p.vp = (const char*)workspace + img;
     p.o = (bf16_t*)o; p.ldo = ldo;
+    p.cos = cos; p.sin = sin;
     p.n_tokens = (int)n_tokens; p.n_heads = n_heads;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
     dim3 grid((unsigned)((n_tokens + BMQ - 1) / BMQ), n_heads);
     hipStream_t st = (hipStream_t)stream;
-    if (head_dim == 128) attn_fwd_pipe_kernel<128><<<grid, 512, 0, st>>>(p);
-    else attn_fwd_pipe_kernel<64><<<grid, 512, 0, st>>>(p);
+    // variant 0 = 32 query rows per wave (8 waves, two per SIMD); 1 = 64 query rows per wave (4 waves)
+    if (cdm_get_variant(0) == 1) {
+        if (head_dim == 128) attn_fwd_pipe_kernel<128, 2><<<grid, 256, 0, st>>>(p);
+        else attn_fwd_pipe_kernel<64, 2><<<grid, 256, 0, st>>>(p);
+    } else {
+        if (head_dim == 128) attn_fwd_pipe_kernel<128, 1><<<grid, 512, 0, st>>>(p);
+        else attn_fwd_pipe_kernel<64, 1><<<grid, 512, 0, st>>>(p);
+    }
     return cdm_check_launch("attn_fwd_packed");
 }
 
 extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
-                                     int64_t ldv, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
-                                     int32_t head_dim, void* workspace, int64_t workspace_bytes, void* stream) {
+                                     int64_t ldv, const float* cos, const float* sin, void* o, int64_t ldo,
+                                     int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
     CDM_REQUIRE(q && k && v && o, CDM_ERR_BAD_ARG, "attn_fwd: null pointer");
-    int32_t rc = check_attn_common("attn_fwd", n_tokens, n_heads, head_dim);
+    int32_t rc = check_attn_common("attn_fwd", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
     if (n_tokens == 0) return CDM_OK;
     const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim);
     CDM_REQUIRE(workspace && cdm_aligned16(workspace) && workspace_bytes >= need, CDM_ERR_BAD_ARG,
                 "attn_fwd: workspace of at least %lld bytes required", (long long)need);
-    // validate everything before the first stage is enqueued
+    // validate the second stage's arguments before the first stage is enqueued
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldq >= d && ldk >= d && ldv >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd: row stride smaller than n_heads*head_dim");
-    CDM_REQUIRE(ldk * 64 * 2 < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd: ldk out of range");
     CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(o) && ldq % 8 == 0 &&
                     ldk % 8 == 0 && ldv % 8 == 0 && ldo % 4 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
-    if ((rc = cdm_require_device())) return rc;
-    const int variant = cdm_get_variant(0);
-    if (variant == 0) {
-        if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, workspace, workspace_bytes, n_tokens, n_heads, head_dim, stream)))
-            return rc;
-        return cdm_attn_fwd_packed_bf16(q, ldq, workspace, o, ldo, n_tokens, n_heads, head_dim, stream);
-    }
-    // measurement variants (non-pipelined kernel on row-major K and per-head V^T):
-    // 1 = 8 waves x 32 query rows, 2 = 4 waves x 64 query rows
-    hipStream_t st = (hipStream_t)stream;
-    const int n_pad = (int)pad_tokens(n_tokens);
-    bf16_t* vt = (bf16_t*)((char*)workspace + 2 * image_bytes(n_tokens, n_heads, head_dim));
-    dim3 tgrid(n_pad / 64, n_heads);
-    if (head_dim == 128) transpose_v_kernel<128><<<tgrid, 256, 0, st>>>((const bf16_t*)v, ldv, vt, (int)n_tokens, n_pad);
-    else transpose_v_kernel<64><<<tgrid, 256, 0, st>>>((const bf16_t*)v, ldv, vt, (int)n_tokens, n_pad);
-    if ((rc = cdm_check_launch("attn_fwd(transpose_v)"))) return rc;
-    AttnParams p;
-    p.q = (const bf16_t*)q; p.ldq = ldq;
-    p.k = (const bf16_t*)k; p.ldk = ldk;
-    p.vt = vt;
-    p.o = (bf16_t*)o; p.ldo = ldo;
-    p.n_tokens = (int)n_tokens; p.n_pad = n_pad; p.n_heads = n_heads;
-    p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
-    if (head_dim == 128) {
-        if (variant == 2) launch_attn<128, 2, 4>(p, st);
-        else launch_attn<128, 1, 8>(p, st);
-    } else {
-        if (variant == 2) launch_attn<64, 2, 4>(p, st);
-        else launch_attn<64, 1, 8>(p, st);
-    }
-    return cdm_check_launch("attn_fwd");
+    if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_heads, head_dim,
+                                    stream)))
+        return rc;
+    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, head_dim, stream);
 }

@@ -56,13 +56,16 @@ class DMAttnProcessor:
     attention over the joint sequence, per-branch output projection (optionally fused with the gated
     residual).
 
-    ``rope_in_gemm_epilogue`` selects where mRoPE is applied: inside the QKV GEMM epilogue (on the fp32
-    accumulators) or by the streaming in-place kernel right after a plain QKV GEMM.  The second is the default:
-    the rotating epilogue currently costs more GEMM time than the extra 8*N*d bytes of the streaming pass.
+    ``rope`` selects where mRoPE is applied: "in_attention" (default: in registers, to K while the attention
+    entry point re-tiles it and to Q when the attention kernel loads it - no extra pass over memory),
+    "gemm_epilogue" (on the fp32 accumulators of the QKV GEMM) or "streaming" (the in-place kernel after a plain
+    QKV GEMM).
     """
 
-    def __init__(self, rope_in_gemm_epilogue: bool = False):
-        self.rope_in_gemm_epilogue = rope_in_gemm_epilogue
+    def __init__(self, rope: str = "in_attention"):
+        if rope not in ("in_attention", "gemm_epilogue", "streaming"):
+            raise ValueError(f"unknown rope placement {rope!r}")
+        self.rope = rope
 
     def __call__(self, attn: "DMAttention", hidden_states: torch.Tensor,
                  encoder_hidden_states: Optional[torch.Tensor] = None, attention_mask: Optional[torch.Tensor] = None,
@@ -95,14 +98,19 @@ class DMAttnProcessor:
         qkv = ws.qkv if ws is not None else torch.empty((n, 3 * d), dtype=torch.bfloat16, device=x.device)
         o = ws.attn_out if ws is not None else torch.empty((n, d), dtype=torch.bfloat16, device=x.device)
 
-        if self.rope_in_gemm_epilogue:
+        wsb = ws.attn_ws if ws is not None else None
+        q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
+        if self.rope == "gemm_epilogue":
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
                          rope_cols=2 * d, head_dim=attn.head_dim)
+            ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb)
         else:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
-            ops.mrope_qk_(qkv[:, :d], qkv[:, d:2 * d], cos, sin, attn.n_heads, attn.head_dim)
-        ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], attn.n_heads, attn.head_dim, out=o,
-                      workspace=ws.attn_ws if ws is not None else None)
+            if self.rope == "streaming":
+                ops.mrope_qk_(q, k, cos, sin, attn.n_heads, attn.head_dim)
+                ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb)
+            else:     # in registers, inside the attention kernels
+                ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin)
         if attn.fp8:
             oq, so = ops.quant_rows(o)
         else:
@@ -235,9 +243,8 @@ class DMBlock(nn.Module):
         yq = torch.empty(x.shape, dtype=ops.FP8_DTYPE, device=x.device)
         st = torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)
         for (s0, ln, b, modulated) in segments:
-            q, s = ops.adaln_rmsnorm_quant(x[s0:s0 + ln], weights[b], shift if modulated else None,
-                                           scale if modulated else None, self.eps)
-            yq[s0:s0 + ln].copy_(q); st[s0:s0 + ln].copy_(s)
+            ops.adaln_rmsnorm_quant(x[s0:s0 + ln], weights[b], shift if modulated else None,
+                                    scale if modulated else None, self.eps, out_q=yq[s0:s0 + ln], out_s=st[s0:s0 + ln])
         return yq, st
 
     def forward(self, hidden_states: torch.Tensor, temb: torch.Tensor,

@@ -45,13 +45,8 @@ def _f32vec(t: Optional[torch.Tensor], name: str, n: int) -> int:
     return _chk(t.reshape(-1), name)
 
 
-_ATTN_VARIANT = [0]
-
-
 def set_variant(op: str, variant: int) -> int:
     lib = _lib.load()
-    if op == "attn":
-        _ATTN_VARIANT[0] = int(variant)
     prev = lib.cdm_set_variant(op.encode(), int(variant))
     if prev < 0:
         raise RuntimeError(f"set_variant failed: {_lib.last_error()}")
@@ -77,17 +72,21 @@ def adaln_rmsnorm(x: torch.Tensor, w: torch.Tensor, shift: Optional[torch.Tensor
     return out
 
 
-def adaln_rmsnorm_quant(x, w, shift=None, scale=None, eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:
+def adaln_rmsnorm_quant(x, w, shift=None, scale=None, eps: float = 1e-6, out_q: Optional[torch.Tensor] = None,
+                        out_s: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Same norm, output quantised per token to e4m3: returns (yq [n, d] float8_e4m3fn, s_tok [n] fp32)."""
     lib = _lib.load()
     n, d = x.shape
     if not x.is_contiguous():
         raise ValueError("x must be contiguous")
-    yq = torch.empty((n, d), dtype=FP8_DTYPE, device=x.device)
-    s = torch.empty((n,), dtype=torch.float32, device=x.device)
+    yq = torch.empty((n, d), dtype=FP8_DTYPE, device=x.device) if out_q is None else out_q
+    s = torch.empty((n,), dtype=torch.float32, device=x.device) if out_s is None else out_s
+    if yq.shape != (n, d) or not yq.is_contiguous() or s.shape != (n,) or not s.is_contiguous():
+        raise ValueError("out_q / out_s must be contiguous [n, d] e4m3 and [n] fp32")
     rc = lib.cdm_adaln_rmsnorm_quant_e4m3(_chk(x, "x", torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
-                                          _f32vec(shift, "shift", d), _f32vec(scale, "scale", d), yq.data_ptr(),
-                                          s.data_ptr(), n, d, float(eps), _stream())
+                                          _f32vec(shift, "shift", d), _f32vec(scale, "scale", d),
+                                          _chk(yq, "out_q", FP8_DTYPE, 2), _chk(s, "out_s", torch.float32, 1), n, d,
+                                          float(eps), _stream())
     _lib.check(rc, "cdm_adaln_rmsnorm_quant_e4m3")
     return yq, s
 
@@ -205,8 +204,10 @@ def attn_workspace_bytes(n_tokens: int, n_heads: int, head_dim: int) -> int:
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
-              out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Full non-causal attention; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free)."""
+              out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+              cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Full non-causal attention; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free).
+    With cos/sin ([n, head_dim/2] fp32) rotate-half mRoPE is applied to Q and K inside the kernels."""
     lib = _lib.load()
     n = q.shape[0]
     d = n_heads * head_dim
@@ -217,20 +218,22 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     need = attn_workspace_bytes(n, n_heads, head_dim)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    half = head_dim // 2
     qp, kp, vp = _chk(q, "q", torch.bfloat16, 2), _chk(k, "k", torch.bfloat16, 2), _chk(v, "v", torch.bfloat16, 2)
     op, wp = _chk(out, "out", torch.bfloat16, 2), _chk(workspace, "workspace", torch.uint8, 1)
-    if _ATTN_TIMER is None or _ATTN_VARIANT[0] != 0:
-        rc = lib.cdm_attn_fwd_bf16(qp, q.stride(0), kp, k.stride(0), vp, v.stride(0), op, out.stride(0), n, n_heads,
-                                   head_dim, wp, workspace.numel(), _stream())
+    cp, sp = _f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half)
+    if _ATTN_TIMER is None:
+        rc = lib.cdm_attn_fwd_bf16(qp, q.stride(0), kp, k.stride(0), vp, v.stride(0), cp, sp, op, out.stride(0), n,
+                                   n_heads, head_dim, wp, workspace.numel(), _stream())
         _lib.check(rc, "cdm_attn_fwd_bf16")
         return out
     # timed form: the same two stages, with HIP events around the attention kernel alone
-    rc = lib.cdm_attn_pack_kv_bf16(kp, k.stride(0), vp, v.stride(0), wp, workspace.numel(), n, n_heads, head_dim,
-                                   _stream())
+    rc = lib.cdm_attn_pack_kv_bf16(kp, k.stride(0), vp, v.stride(0), cp, sp, wp, workspace.numel(), n, n_heads,
+                                   head_dim, _stream())
     _lib.check(rc, "cdm_attn_pack_kv_bf16")
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    rc = lib.cdm_attn_fwd_packed_bf16(qp, q.stride(0), wp, op, out.stride(0), n, n_heads, head_dim, _stream())
+    rc = lib.cdm_attn_fwd_packed_bf16(qp, q.stride(0), cp, sp, wp, op, out.stride(0), n, n_heads, head_dim, _stream())
     e1.record()
     _lib.check(rc, "cdm_attn_fwd_packed_bf16")
     _ATTN_TIMER.append((e0, e1))

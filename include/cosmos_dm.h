@@ -128,31 +128,34 @@ int32_t cdm_mrope_qk_bf16(void* q, int64_t ldq, void* k, int64_t ldk, const floa
                           int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream);
 
 /*
- * Shared full (non-causal) self-attention over the joint sequence - replaces the attention
- * processor's scaled_dot_product_attention call (README.md:74; eager form transformers
- * models/qwen3_vl/modeling_qwen3_vl.py:171-193, fp32 softmax).
- *   O = softmax(Q K^T / sqrt(head_dim)) V per head, no mask.
+ * Shared full (non-causal) self-attention over the joint sequence, with rotate-half mRoPE applied in
+ * registers to Q and K on the way in - replaces the attention processor's apply_rotary_pos_emb +
+ * scaled_dot_product_attention (README.md:74; eager form transformers
+ * models/qwen3_vl/modeling_qwen3_vl.py:171-193 with fp32 softmax; RoPE :138-142, :412-435).
+ *   O = softmax(rope(Q) rope(K)^T / sqrt(head_dim)) V per head, no mask.
  *   q, k, v: [n_tokens, n_heads, head_dim] with row strides ldq, ldk, ldv; o: [n_tokens, n_heads*head_dim] (ldo).
+ *   cos, sin: [n_tokens, head_dim/2] fp32 rotary tables, or both null when Q and K are already rotated.
  *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds K and V re-laid
  *   out as 64-key tile images); its contents are undefined afterwards.
  * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
  */
 int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim);
 int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
-                          void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
-                          void* workspace, int64_t workspace_bytes, void* stream);
+                          const float* cos, const float* sin, void* o, int64_t ldo, int64_t n_tokens,
+                          int32_t n_heads, int32_t head_dim, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
- * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first K and V
- * are packed into the workspace as tile images (a streaming pass), then the attention kernel proper
- * reads Q and the workspace.  A caller that times or profiles the attention kernel alone, or that
- * reuses packed K/V across calls, uses these.
+ * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first K (rotated
+ * if tables are given) and V are packed into the workspace as tile images (a streaming pass), then the
+ * attention kernel proper reads Q (rotating it with the same tables) and the workspace.  A caller that
+ * times or profiles the attention kernel alone, or that reuses packed K/V across calls, uses these.
  */
-int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, void* workspace,
-                              int64_t workspace_bytes, int64_t n_tokens, int32_t n_heads, int32_t head_dim,
-                              void* stream);
-int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const void* workspace, void* o, int64_t ldo,
-                                 int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream);
+int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
+                              const float* sin, void* workspace, int64_t workspace_bytes, int64_t n_tokens,
+                              int32_t n_heads, int32_t head_dim, void* stream);
+int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
+                                 const void* workspace, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
+                                 int32_t head_dim, void* stream);
 
 /*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each

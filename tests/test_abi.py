@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} declared in include/cosmos_dm.h but not exported"
     assert set(names) == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
     assert lib.cdm_version() >= 100
-    assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 3 * 128 * 2 * 64 * 2
+    assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 2 * 128 * 2 * 64 * 2
 
 
 def test_bad_arguments_are_rejected_on_the_host():
@@ -47,14 +47,15 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert g(epi=_lib.EPI_GATE_RESIDUAL) == _lib.ERR_BAD_ARG     # R missing
     assert g(epi=_lib.EPI_ROPE_QK) == _lib.ERR_BAD_ARG           # tables missing
     assert g(lda=100) == _lib.ERR_BAD_ARG                        # stride < K
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, 64, 16, 1, 48, fake, 1 << 20, None) == _lib.ERR_BAD_SHAPE
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, 64, 16, 1, 64, fake, 16, None) == _lib.ERR_BAD_ARG
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 48, fake, 1 << 20, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 64, fake, 16, None) == _lib.ERR_BAD_ARG
     assert "workspace" in _lib.last_error()
     assert lib.cdm_mrope_qk_bf16(fake, 64, None, 0, fake, fake, 4, 1, 32, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_quant_rows_e4m3(fake, 128, fake, fake, 4, 100, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_set_variant(b"nope", 0) == _lib.ERR_BAD_ARG
     # empty inputs are accepted without work
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, 64, 0, 1, 64, None, 0, None) == _lib.OK
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, None, fake, 64, 16, 1, 64, fake, 1 << 20, None) == _lib.ERR_BAD_ARG   # cos without sin
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 0, 1, 64, None, 0, None) == _lib.OK
 
 
 @pytest.mark.skipif(HAS_GPU, reason="needs a host without a GPU")

@@ -54,7 +54,7 @@ def test_c0_single_block_parity():
     assert_close(y2.float().cpu() - xr, want2 - xr, 0.999, BF16_REL, "C0 block update")
 
 
-def test_rope_epilogue_and_streaming_rope_agree():
+def test_rope_placements_agree():
     from cosmos_amd import DMAttnProcessor
     cfg = DMConfig("t", 256, 2, 128, 512, 1, (2, 4, 8), n_text=8)
     blk = make_block(cfg, 5)
@@ -62,10 +62,12 @@ def test_rope_epilogue_and_streaming_rope_agree():
     x, _ = rand_bf16((cfg.n_tokens, 256), g)
     temb, _ = rand_bf16((256,), g)
     st = DMStack(cfg, device=dev())
-    y1 = blk(x, temb, st.rotary(dev()), st.segments())
-    blk.attn.set_processor(DMAttnProcessor(rope_in_gemm_epilogue=True))
-    y2 = blk(x, temb, st.rotary(dev()), st.segments())
-    assert_close(y2, y1.float().cpu(), 0.99999, 4e-3, "rope placement")
+    ys = []
+    for mode in ("in_attention", "gemm_epilogue", "streaming"):
+        blk.attn.set_processor(DMAttnProcessor(rope=mode))
+        ys.append(blk(x, temb, st.rotary(dev()), st.segments()))
+    assert_close(ys[1], ys[0].float().cpu(), 0.99999, 4e-3, "rope in GEMM epilogue vs in attention")
+    assert_close(ys[2], ys[0].float().cpu(), 0.99999, 4e-3, "streaming rope vs in attention")
 
 
 def test_block_gate_zero_is_identity():
@@ -182,10 +184,9 @@ def test_c1_full_size_attention_sampled_rows():
     qkv = (torch.randn((n, 3 * d), generator=g, device=dev()) / (hd ** 0.5)).to(torch.bfloat16)
     pos, _ = rotary.build_positions(0, cfg.grid)
     cos, sin = rotary.rotary_tables(pos, hd, cfg.mrope_sections)
-    pre = qkv.clone()
+    pre = qkv
     q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
-    ops.mrope_qk_(q, k, cos.to(dev()), sin.to(dev()), H, hd)
-    o = ops.attention(q, k, v, H, hd)
+    o = ops.attention(q, k, v, H, hd, cos=cos.to(dev()), sin=sin.to(dev()))      # mRoPE in registers
     torch.cuda.synchronize()
     rows = torch.cat([torch.tensor([0, 1, 31, 32, 255, 256, n - 1, n - 64]),
                       torch.randint(0, n, (56,), generator=torch.Generator().manual_seed(1))])

@@ -154,7 +154,7 @@ def test_grouped_gemm_three_segments():
 
 
 # ------------------------------------------------------------------ attention
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("n,H,hd", [(64, 2, 64), (256, 1, 128), (1000, 3, 128), (321, 2, 64), (1, 1, 128), (130, 2, 128), (65, 1, 64),
                                     (128, 2, 128), (191, 1, 128), (192, 1, 128), (577, 2, 128)])
 def test_attention_vs_oracle(n, H, hd, variant):
@@ -168,6 +168,26 @@ def test_attention_vs_oracle(n, H, hd, variant):
         ops.set_variant("attn", prev)
     want = O.attention(qkvr[:, :d].view(n, H, hd), qkvr[:, d:2 * d].view(n, H, hd), qkvr[:, 2 * d:].view(n, H, hd))
     assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"attention n={n} H={H} hd={hd} variant={variant}")
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n,H,hd,sections", [(300, 2, 128, (32, 48, 48)), (130, 3, 64, (16, 24, 24))])
+def test_attention_with_rope_in_registers(n, H, hd, sections, variant):
+    g = gen(n + hd)
+    d = H * hd
+    pos, _ = rotary.build_positions(n - 7 * 6 * 5 - 4, (7, 6, 5), 4) if n == 300 else rotary.build_positions(10, (4, 5, 6), 0)
+    assert pos.shape[1] == n
+    cos, sin = rotary.rotary_tables(pos, hd, sections)
+    qkv, qkvr = rand_bf16((n, 3 * d), g, 1.5)
+    prev = ops.set_variant("attn", variant)
+    try:
+        o = ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], H, hd, cos=cos.to(dev()), sin=sin.to(dev()))
+    finally:
+        ops.set_variant("attn", prev)
+    qr = O.apply_mrope(qkvr[:, :d].view(n, H, hd), cos, sin)
+    kr = O.apply_mrope(qkvr[:, d:2 * d].view(n, H, hd), cos, sin)
+    want = O.attention(qr, kr, qkvr[:, 2 * d:].view(n, H, hd))
+    assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"attention+rope n={n} hd={hd} variant={variant}")
 
 
 def test_attention_closed_forms_and_determinism():
