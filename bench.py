@@ -20,6 +20,11 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per attention launch (L2 fetches + writes) for the 56,832-token, 32x128-head shape, from two
+# rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a plain streaming
+# kernel of known size (FETCH_SIZE unit = 2 KiB, WRITE_SIZE unit = 1 KiB on this chip).  Counters cannot be read
+# from inside this process, so other shapes report null.
+ATTN_TRAFFIC_BYTES = {(56832, 32, 128): 14.85e9 + 0.614e9}
 
 
 def cpu_baseline(cfg, sample_tokens: int):
@@ -70,6 +75,10 @@ def main():
     ap.add_argument("--rope", default="in_attention", choices=["in_attention", "gemm_epilogue", "streaming"])
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-copy-mib", type=int, default=0,
+                    help="counter calibration aid: after the timed region run ONE plain streaming kernel that reads and "
+                         "writes this many MiB (torch.bitwise_not on int32), so that a rocprofv3 --pmc pass of this "
+                         "command also holds FETCH_SIZE / WRITE_SIZE for a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -116,6 +125,13 @@ def main():
     wall = time.perf_counter() - t0
     events = ops.time_attention(False)
     assert bool(torch.isfinite(out.float()).all()), "non-finite output"
+    if args.pmc_copy_mib:
+        src = torch.zeros(args.pmc_copy_mib << 18, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.bitwise_not(src, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     ms_per_step = wall * 1e3 / args.steps
     attn_ms = [a.elapsed_time(b) for a, b in events]
@@ -137,7 +153,9 @@ def main():
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
                    "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
-                     "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4),
+                     "traffic": ATTN_TRAFFIC_BYTES.get((cfg.n_tokens, cfg.n_heads, cfg.head_dim))
+                     if args.attn_variant == 0 else None,
                      "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},
         "extra": {"ms_per_block": round(ms_per_step / cfg.n_blocks, 3),
                   "non_attention_ms_per_block": round(gemm_ms_per_block, 3),
