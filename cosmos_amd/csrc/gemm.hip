@@ -297,7 +297,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 // ---------------------------------------------------------------------------------------------
 constexpr int kStageBytes4 = BM * 64;   // 16 KB per operand per stage
 
-__device__ __forceinline__ int swz4(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
+// XOR swizzle of the four 16-byte chunks of a 64-byte ring row.  The LDS serves a 16-byte-per-lane read in four
+// passes of 16 lanes: {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of each half-wave (measured with a
+// two-lane probe).  A fragment read has one chunk index per half-wave and row = lane % 32, so within a pass the 16
+// rows must cover the sixteen slots (row % 4, chunk ^ swz) of the 256-byte bank window: the four rows of a pass that
+// share row % 4 have row / 4 in {0, 3, 5, 6} or in {1, 2, 4, 7}, and (row / 8) % 4 separates both sets.
+__device__ __forceinline__ int swz4(int row) { return (row >> 3) & 3; }
 
 __device__ __forceinline__ bf16x8 lds_frag4(const char* tile, int row, int chunk) {
     return *reinterpret_cast<const bf16x8*>(tile + row * 64 + ((chunk ^ swz4(row)) << 4));
@@ -310,10 +315,10 @@ struct Frags {
 
 // k-step `ks` (0 or 1) of the stage at `sa`/`sb`.  bf16: chunk 2ks + kh.  e4m3: the stage is ONE 64-element MFMA
 // step whose operand is the chunk pair (2kh, 2kh+1); "ks" then selects the low or the high chunk of the pair.
-__device__ __forceinline__ void load_frags(Frags& f, const char* sa, const char* sb, int ks, int wm, int wn, int lane,
-                                           bool fp8) {
+template <bool FP8>
+__device__ __forceinline__ void load_frags(Frags& f, const char* sa, const char* sb, int ks, int wm, int wn, int lane) {
     const int r32 = lane & 31, kh = lane >> 5;
-    const int chunk = fp8 ? 2 * kh + ks : 2 * ks + kh;
+    const int chunk = FP8 ? 2 * kh + ks : 2 * ks + kh;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) f.a[mi] = lds_frag4(sa, wm * 128 + mi * 32 + r32, chunk);
 #pragma unroll
@@ -432,15 +437,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     issue(0, 0); issue(1, 1); issue(2, 2); issue(3, 3);
     asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");     // tile 0 has landed everywhere
     Frags X, Y;
-    load_frags(X, s_a, s_b, 0, wm, wn, lane, FP8);
+    load_frags<FP8>(X, s_a, s_b, 0, wm, wn, lane);
 
 #define CDM_STAGE(T, SLOT, NEXT)                                                                                  \
-    load_frags(Y, s_a + (SLOT) * kStageBytes4, s_b + (SLOT) * kStageBytes4, 1, wm, wn, lane, FP8);                \
+    load_frags<FP8>(Y, s_a + (SLOT) * kStageBytes4, s_b + (SLOT) * kStageBytes4, 1, wm, wn, lane);                     \
     if (!FP8) mma_bf16(X, acc);                                                                                   \
     else { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); mma_fp8(X, Y, acc, 0, 2); }                         \
     asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                     \
     if (!FP8) { issue((T) + 4, SLOT); } else { mma_fp8(X, Y, acc, 2, 4); issue((T) + 4, SLOT); }                  \
-    load_frags(X, s_a + (NEXT) * kStageBytes4, s_b + (NEXT) * kStageBytes4, 0, wm, wn, lane, FP8);                \
+    load_frags<FP8>(X, s_a + (NEXT) * kStageBytes4, s_b + (NEXT) * kStageBytes4, 0, wm, wn, lane);                     \
     if (!FP8) mma_bf16(Y, acc);
     for (int kt = 0; kt < KT; kt += 4) {
         CDM_STAGE(kt, 0, 1)
