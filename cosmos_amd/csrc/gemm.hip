@@ -10,9 +10,12 @@
 // Global -> LDS goes through the direct-to-LDS path (global_load_lds_dwordx4): each wave
 // instruction deposits 64 x 16 B = 8 tile rows linearly in LDS; bank conflicts are avoided by
 // permuting which 16-byte chunk of a row each lane fetches (XOR swizzle on the source side).
-// Two LDS stages (2 x 64 KB): the loads of k-tile t+1 are in flight while k-tile t is multiplied.
+// Two pipelines share tile, swizzle idea and epilogues: a two-stage one (2 x 64 KB of LDS: the loads of k-tile
+// t+1 are in flight while k-tile t is multiplied) and the default five-slot ring further down.
 // Workgroup ids are remapped so that each XCD (ids are dealt round-robin over the 8 XCDs) works
 // on a compact block of tiles and its private L2 sees the reuse.
+#include <type_traits>
+
 #include "cdm_common.h"
 
 namespace {
@@ -288,91 +291,43 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 }
 
 // ---------------------------------------------------------------------------------------------
-// Deep pipeline: same 256x256 tile and wave layout, but k-tiles of 64 BYTES and FOUR LDS stages
-// (4 x 32 KB), so the loads of k-tiles t+1 .. t+3 are in flight while k-tile t is multiplied
-// (about three stage times of latency tolerance instead of one).  A wave waits only for its own
-// loads of tile t (s_waitcnt vmcnt(16): the 2 x 8 younger loads may stay outstanding) before the
-// workgroup barrier.  Rows are 64 bytes = 4 chunks; chunk c of row r sits at position
-// c ^ (((r >> 1) ^ (r >> 3)) & 3), which keeps 8 and 16 consecutive lanes on distinct banks.
+// Ring pipeline (default): 256x256 tile, 4 waves, 128-byte tile rows (k-tiles of 64 bf16 / 128 e4m3 elements) and a
+// five-slot ring of single-operand granules.
+//  * A direct-to-LDS load instruction that covers 8 rows x 128 bytes (whole cache lines) costs the vector L1 about
+//    40 % less time per byte than one that covers 16 rows x 64 bytes, and with 256x256 tiles the L1 path is what
+//    the pipeline competes for.  160 KB of LDS hold five 32 KB granules (256 rows x 128 B of A or of W): granule
+//    g = 2t + (0: A, 1: W) of k-tile t lives in slot g % 5, so two slots are being read and three are landing.
+//  * stage t (bf16):  P0 P1 P2 | wait + barrier | P3      Pk = the 16 MFMAs of k-step k; the fragments of the next
+//    stage t (e4m3):  P0 | wait + barrier | P1            k-step are read under the first eight of them.
+//    The barrier says "every wave has finished reading tile t, and tile t+1 has landed"; it releases the two slots
+//    of tile t.  W(t+2), needed at the next barrier, goes out at once (one load after every second MFMA of the last
+//    phase); A(t+3) follows spread over the phases before the next barrier.
+//  * The instruction order inside a stage is pinned with scheduling fences: a wave that issues its loads back to
+//    back sits in the vector-memory issue queue for hundreds of cycles (all four waves do so at the same moment)
+//    and with one wave per SIMD nothing else feeds the matrix pipe meanwhile; one load per few MFMAs is covered by
+//    MFMAs already queued.
+//  * The loop body is ONE stage; the slot numbers live in scalar registers and rotate by renaming.  (A loop
+//    unrolled over the five-stage period needs mid-loop exits, and the spill reloads the compiler then places at
+//    the loop head wait with vmcnt(0), which drains every direct-to-LDS load in flight.)
 // ---------------------------------------------------------------------------------------------
-constexpr int kStageBytes4 = BM * 64;   // 16 KB per operand per stage
+constexpr int kGranule = BM * 128;      // 32 KB
 
-// XOR swizzle of the four 16-byte chunks of a 64-byte ring row.  The LDS serves a 16-byte-per-lane read in four
-// passes of 16 lanes: {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of each half-wave (measured with a
-// two-lane probe).  A fragment read has one chunk index per half-wave and row = lane % 32, so within a pass the 16
-// rows must cover the sixteen slots (row % 4, chunk ^ swz) of the 256-byte bank window: the four rows of a pass that
-// share row % 4 have row / 4 in {0, 3, 5, 6} or in {1, 2, 4, 7}, and (row / 8) % 4 separates both sets.
-__device__ __forceinline__ int swz4(int row) { return (row >> 3) & 3; }
+// chunk swizzle of a 128-byte ring row; a function of row % 32 only, so that the fragment address of row block mi
+// is the lane's address plus a constant.  The LDS serves a 16-byte-per-lane read in four passes of 16 lanes:
+// {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of each half-wave (measured with a two-lane probe); within
+// a pass the chunk index is the same for all lanes and row = lane % 32, and this swizzle puts the 16 rows of either
+// pass on the 16 distinct 16-byte slots of the 256-byte bank window.
+__device__ __forceinline__ int swz128(int row) { return (row ^ ((row & 31) >> 3)) & 7; }
 
-__device__ __forceinline__ bf16x8 lds_frag4(const char* tile, int row, int chunk) {
-    return *reinterpret_cast<const bf16x8*>(tile + row * 64 + ((chunk ^ swz4(row)) << 4));
-}
-
-// fragments of one 16-element (bf16) / 64-element (e4m3, two chunks) k-step of a stage: 4 A + 4 W
+template <bool FP8>
 struct Frags {
-    bf16x8 a[4], b[4];
+    using T = typename std::conditional<FP8, i32x8, bf16x8>::type;
+    T a[4], b[4];
 };
 
-// k-step `ks` (0 or 1) of the stage at `sa`/`sb`.  bf16: chunk 2ks + kh.  e4m3: the stage is ONE 64-element MFMA
-// step whose operand is the chunk pair (2kh, 2kh+1); "ks" then selects the low or the high chunk of the pair.
-template <bool FP8>
-__device__ __forceinline__ void load_frags(Frags& f, const char* sa, const char* sb, int ks, int wm, int wn, int lane) {
-    const int r32 = lane & 31, kh = lane >> 5;
-    const int chunk = FP8 ? 2 * kh + ks : 2 * ks + kh;
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) f.a[mi] = lds_frag4(sa, wm * 128 + mi * 32 + r32, chunk);
-#pragma unroll
-    for (int ni = 0; ni < 4; ++ni) f.b[ni] = lds_frag4(sb, wn * 128 + ni * 32 + r32, chunk);
-}
-
-__device__ __forceinline__ void mma_bf16(const Frags& f, f32x16 (&acc)[4][4]) {
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[mi], f.b[ni], acc[mi][ni], 0, 0, 0);
-}
-
-__device__ __forceinline__ void mma_fp8(const Frags& lo, const Frags& hi, f32x16 (&acc)[4][4], int mi_begin,
-                                        int mi_end) {
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-        if (mi < mi_begin || mi >= mi_end) continue;
-        const int4 al = __builtin_bit_cast(int4, lo.a[mi]), ah = __builtin_bit_cast(int4, hi.a[mi]);
-        const i32x8 av = {al.x, al.y, al.z, al.w, ah.x, ah.y, ah.z, ah.w};
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni) {
-            const int4 bl = __builtin_bit_cast(int4, lo.b[ni]), bh = __builtin_bit_cast(int4, hi.b[ni]);
-            const i32x8 bv = {bl.x, bl.y, bl.z, bl.w, bh.x, bh.y, bh.z, bh.w};
-            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                          0x7f7f7f7f);
-        }
-    }
-}
-
-__device__ __forceinline__ void issue_loads4(const char* abase, const char* wbase, const char* w2base,
-                                             const uint32_t (&oa)[4], const uint32_t (&ob)[4], uint32_t w2mask,
-                                             uint32_t la, uint32_t lb) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        lds_dma16(abase, oa[i], la + i * 4096);
-        const char* wb = ((w2mask >> i) & 1u) ? w2base : wbase;   // wave-uniform choice
-        lds_dma16(wb, ob[i], lb + i * 4096);
-    }
-}
-
-// Schedule of one stage T (ring slot T & 3), with the fragments X of its first k-step already in registers:
-//     Y <- fragments of the second k-step                       (LDS reads fly under the next MFMAs)
-//     16 MFMAs on X
-//     wait: own Y reads done (this wave no longer needs slot T), tile T+1 landed; workgroup barrier
-//     refill slot T with tile T+4; X <- first k-step of tile T+1  (LDS reads fly under the next MFMAs)
-//     16 MFMAs on Y
-// so the matrix pipe always has queued work while LDS and global latencies are being paid, and the barrier
-// sits in the middle of a stage instead of in front of a fragment-read bubble.
 template <int EPI, bool FP8>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel4(const GemmParams p) {
-    __shared__ __attribute__((aligned(1024))) char s_a[4 * kStageBytes4];
-    __shared__ __attribute__((aligned(1024))) char s_b[4 * kStageBytes4];
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_ring_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(1024))) char s_ring[5 * kGranule];
 
     const int total = p.tiles_m * p.tiles_n;
     const int per_xcd = (total + 7) >> 3;
@@ -392,31 +347,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int m0 = tm * BM;
     const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
 
-    // per-lane byte offsets of the 4 + 4 loads of one k-tile (each instruction = 16 tile rows of 64 bytes)
-    uint32_t oa[4], ob[4];
-    uint32_t w2mask = 0;
+    // per-lane byte offsets of the 8 + 8 loads of one k-tile (each instruction = 8 tile rows of 128 bytes)
+    uint32_t oa[8], ob[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = (i * 4 + wave) * 16 + (lane >> 2);
-        const int chunk = (lane & 3) ^ swz4(row);
+    for (int j = 0; j < 8; ++j) {
+        const int row = (j * 4 + wave) * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ swz128(row);
         int am = row;
         am = (m0 + am) < p.M ? am : p.M - 1 - m0;
-        oa[i] = (uint32_t)(am * (int)p.lda + chunk * 16);
-        int bn;
-        if (EPI == CDM_EPI_SWIGLU) {
-            const int grp = ((i * 4 + wave) * 16) >> 6;      // wave-uniform
-            if (grp & 1) w2mask |= 1u << i;
-            bn = (grp >> 1) * 64 + (row & 63);
-        } else {
-            bn = row;
-        }
+        oa[j] = (uint32_t)(am * (int)p.lda + chunk * 16);
+        // SWIGLU: tile rows come in 64-row groups [gate | up | gate | up]; the rows of load j lie in group j / 2
+        int bn = (EPI == CDM_EPI_SWIGLU) ? (j >> 2) * 64 + (row & 63) : row;
         bn = (n0 + bn) < p.N ? bn : p.N - 1 - n0;
-        ob[i] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
+        ob[j] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
     }
     const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
     const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)n0 * p.ldw;
     const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)n0 * p.ldw : wbase;
-    const uint32_t la = lds_addr_of(s_a) + wave * 1024, lb = lds_addr_of(s_b) + wave * 1024;
+    const uint32_t l0 = lds_addr_of(s_ring) + wave * 1024;
 
     f32x16 acc[4][4];
 #pragma unroll
@@ -426,34 +374,102 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
-    const int KT = p.K / (FP8 ? 64 : 32);   // k-tiles of 64 bytes; a multiple of 4 (host-checked)
-    // tile index clamped to the last one: every stage issues the same 8 loads per wave, which keeps the
-    // s_waitcnt vmcnt(16) below valid up to the end (the surplus loads rewrite a free slot with the last tile)
-    auto issue = [&](int t, int slot) {
-        const int ko = (t < KT ? t : KT - 1) * 64;
-        issue_loads4(abase + ko, wbase + ko, w2base + ko, oa, ob, w2mask, la + slot * kStageBytes4,
-                     lb + slot * kStageBytes4);
+    const int KT = p.K / (FP8 ? 128 : 64);   // k-tiles of 128 bytes (at least 2, host-checked)
+    // load j (0..7) of the A (op = 0) or W (op = 1) granule of k-tile t into `slot`.  The tile index is clamped to
+    // the last one so that the number of loads per stage, and with it the vmcnt arithmetic, is the same to the end
+    // (a surplus load rewrites a free slot).
+    auto gload = [&](int t, int op, int slot, int j) {
+        const int ko = (t < KT ? t : KT - 1) * 128;
+        if (op == 0) {
+            lds_dma16(abase + ko, oa[j], l0 + slot * kGranule + j * 4096);
+        } else {
+            const char* wb = (EPI == CDM_EPI_SWIGLU && ((j >> 1) & 1)) ? w2base : wbase;
+            lds_dma16(wb + ko, ob[j], l0 + slot * kGranule + j * 4096);
+        }
     };
-    issue(0, 0); issue(1, 1); issue(2, 2); issue(3, 3);
-    asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");     // tile 0 has landed everywhere
-    Frags X, Y;
-    load_frags<FP8>(X, s_a, s_b, 0, wm, wn, lane);
-
-#define CDM_STAGE(T, SLOT, NEXT)                                                                                  \
-    load_frags<FP8>(Y, s_a + (SLOT) * kStageBytes4, s_b + (SLOT) * kStageBytes4, 1, wm, wn, lane);                     \
-    if (!FP8) mma_bf16(X, acc);                                                                                   \
-    else { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); mma_fp8(X, Y, acc, 0, 2); }                         \
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                     \
-    if (!FP8) { issue((T) + 4, SLOT); } else { mma_fp8(X, Y, acc, 2, 4); issue((T) + 4, SLOT); }                  \
-    load_frags<FP8>(X, s_a + (NEXT) * kStageBytes4, s_b + (NEXT) * kStageBytes4, 0, wm, wn, lane);                     \
-    if (!FP8) mma_bf16(Y, acc);
-    for (int kt = 0; kt < KT; kt += 4) {
-        CDM_STAGE(kt, 0, 1)
-        CDM_STAGE(kt + 1, 1, 2)
-        CDM_STAGE(kt + 2, 2, 3)
-        CDM_STAGE(kt + 3, 3, 0)
+    const int r32 = lane & 31, kh = lane >> 5;
+    constexpr int KS = FP8 ? 2 : 4;     // MFMA k-steps per k-tile
+    // per-lane byte offset of the fragment of k-step ks in row block 0 of the wave's half.  bf16: chunk 2ks + kh;
+    // e4m3: the 32 bytes of chunks (4ks + 2kh, 4ks + 2kh + 1), which the swizzle keeps adjacent (position ^ 1).
+    uint32_t fa[KS], fb[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int chunk = FP8 ? 4 * ks + 2 * kh : 2 * ks + kh;
+        const uint32_t in_row = (uint32_t)(r32 * 128 + ((chunk ^ swz128(r32)) << 4));
+        fa[ks] = in_row + wm * 16384;
+        fb[ks] = in_row + wn * 16384;
     }
-#undef CDM_STAGE
+    auto rd = [&](uint32_t off) {
+        if constexpr (FP8) {
+            const int4 lo = *reinterpret_cast<const int4*>(s_ring + off);
+            const int4 hi = *reinterpret_cast<const int4*>(s_ring + (off ^ 16));
+            return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        } else {
+            return *reinterpret_cast<const bf16x8*>(s_ring + off);
+        }
+    };
+    // fragment q of k-step ks: q = 0 -> a0, 1..4 -> b0..b3, 5..7 -> a1..a3 (the order the MFMAs need them)
+    auto frag = [&](Frags<FP8>& f, int slot_a, int slot_b, int ks, int q) {
+        if (q == 0) f.a[0] = rd(fa[ks] + slot_a * kGranule);
+        else if (q <= 4) f.b[q - 1] = rd(fb[ks] + slot_b * kGranule + (q - 1) * 4096);
+        else f.a[q - 4] = rd(fa[ks] + slot_a * kGranule + (q - 4) * 4096);
+    };
+    auto mfma = [&](const Frags<FP8>& f, int i) {
+        const int mi = i >> 2, ni = i & 3;
+        if constexpr (FP8)
+            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[mi], f.b[ni], acc[mi][ni], 0 /*A: e4m3*/,
+                                                                          0 /*B: e4m3*/, 0, 0x7f7f7f7f /*2^0*/, 0,
+                                                                          0x7f7f7f7f);
+        else
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[mi], f.b[ni], acc[mi][ni], 0, 0, 0);
+    };
+    // prologue: granules 0..3 (tiles 0 and 1)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) gload(0, 0, 0, j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) gload(0, 1, 1, j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) gload(1, 0, 2, j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) gload(1, 1, 3, j);
+    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");     // tile 0 has landed everywhere
+    Frags<FP8> X, Y;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) frag(X, 0, 1, 0, q);
+
+#define CDM_FENCE __builtin_amdgcn_sched_barrier(0)
+// one k-step: 16 MFMAs on CUR, the 8 fragment reads of (FA, FB, FKS) into NXT under the first eight, and the
+// statement LOADS (a function of the MFMA index i) after each MFMA
+#define CDM_KSTEP(CUR, NXT, FA, FB, FKS, LOADS)                                                                   \
+    _Pragma("unroll") for (int i = 0; i < 16; ++i) {                                                              \
+        mfma(CUR, i);                                                                                             \
+        if (i < 8) frag(NXT, FA, FB, FKS, i);                                                                     \
+        LOADS;                                                                                                    \
+        CDM_FENCE;                                                                                                \
+    }
+#define CDM_RING_BARRIER                                                                                          \
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                      \
+    CDM_FENCE;
+    // slots: tile t -> ((2t) % 5, (2t+1) % 5); A(t+2) -> (2t+4) % 5 = the fifth slot; W(t+2) -> slot of A(t)
+    int sa = 0, sb = 1, na = 2, nb = 3, f2 = 4;
+    for (int t = 0; t < KT; ++t) {
+        if constexpr (FP8) {
+            CDM_KSTEP(X, Y, sa, sb, 1, if (i & 1) gload(t + 2, 0, f2, i >> 1))
+            CDM_RING_BARRIER
+            CDM_KSTEP(Y, X, na, nb, 0, if (i & 1) gload(t + 2, 1, sa, i >> 1))
+        } else {
+            CDM_KSTEP(X, Y, sa, sb, 1, if (i == 5 || i == 11) gload(t + 2, 0, f2, i == 5 ? 0 : 1))
+            CDM_KSTEP(Y, X, sa, sb, 2, if (i == 1 || i == 7 || i == 13) gload(t + 2, 0, f2, i == 1 ? 2 : i == 7 ? 3 : 4))
+            CDM_KSTEP(X, Y, sa, sb, 3, if (i == 3 || i == 9 || i == 15) gload(t + 2, 0, f2, i == 3 ? 5 : i == 9 ? 6 : 7))
+            CDM_RING_BARRIER
+            CDM_KSTEP(Y, X, na, nb, 0, if (i & 1) gload(t + 2, 1, sa, i >> 1))
+        }
+        const int o_sa = sa, o_sb = sb;
+        sa = na; sb = nb; na = f2; nb = o_sa; f2 = o_sb;
+    }
+#undef CDM_RING_BARRIER
+#undef CDM_KSTEP
+#undef CDM_FENCE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // surplus loads must not outlive the workgroup's LDS
     epilogue<EPI, FP8>(p, acc, m0, n0, wm, wn, lane);
 }
@@ -498,12 +514,10 @@ int32_t run(GemmParams& p, int64_t M, int64_t N, int32_t epilogue, hipStream_t s
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    // variant 0 = tuned default (bf16: four-slot ring pipeline; e4m3: two-stage pipeline, which measures ~1.5x
-    // faster for the 64-element MFMA step); 1 = two-stage; 2 = four-slot ring
-    const int variant = cdm_get_variant(1);
-    const bool deep = variant == 2 || (variant == 0 && !FP8);
+    // variant 0 = ring pipeline (default); 1 = two-stage pipeline
+    const bool ring = cdm_get_variant(1) != 1;
 #define CDM_LAUNCH(E)                                                         \
-    if (deep) gemm_kernel4<E, FP8><<<grid, kThreads, 0, st>>>(p);             \
+    if (ring) gemm_ring_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p);         \
     else gemm_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p)
     switch (epilogue) {
         case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;
