@@ -100,9 +100,9 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 
 // One pipeline step.  Everything the first MFMAs need is already in registers when the workgroup barrier at
 // the top of the step releases the wave, and all softmax arithmetic is placed under MFMAs:
-//   block A  : S(j+1) = K(j+1) Q^T, 16 MFMAs starting from literal zero (rolling K fragment window, first
+//   block A  : S(j+1) = K(j+1) Q^T - m_ref, 16 MFMAs seeded with -m_ref (rolling K fragment window, first
 //              KWIN k-steps preloaded in the previous step)
-//              ||  p = exp2(s_cur - m_ref), bf16 pack, row sum of tile j ; first V^T fragments of tile j
+//              ||  p = exp2(s_cur), bf16 pack, row sum of tile j ; first V^T fragments of tile j
 //   block B  : O^T += V^T P^T, 16 MFMAs (rolling V^T window)
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
@@ -111,20 +111,19 @@ template <int HD, int QS>
 __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
-                                          f32x16 (&oacc)[QS][HD / 32], float (&m_ref)[QS], float (&l_run)[QS], int lane,
+                                          f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
                                           bool next_ragged, int next_keys_valid) {
     constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
     // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot and
     // their result is never used - cheaper than a second copy of the step.)
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
         for (int qs = 0; qs < QS; ++qs) {
             s_next[qs][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][0], qf[qs][ks],
-                                                                    ks == 0 ? zero : s_next[qs][0], 0, 0, 0);
+                                                                    ks == 0 ? negm[qs] : s_next[qs][0], 0, 0, 0);
             s_next[qs][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][1], qf[qs][ks],
-                                                                    ks == 0 ? zero : s_next[qs][1], 0, 0, 0);
+                                                                    ks == 0 ? negm[qs] : s_next[qs][1], 0, 0, 0);
         }
         if (ks + KWIN < KS) {
             kw[ks % KWIN][0] = k_frag<HD>(sk_next, ks + KWIN, 0, lane);
@@ -142,8 +141,8 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
                 bf16x2 pp;
-                pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e] - m_ref[qs]);
-                pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1] - m_ref[qs]);
+                pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e]);
+                pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1]);
                 psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
                 p8[e] = pp[0];
                 p8[e + 1] = pp[1];
@@ -194,18 +193,24 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // ---- tail
+    // ---- tail.  mx is relative to the reference (the scores are); moving the reference by d means: O and l
+    // shrink by 2^-d, the scores already computed for tile j+1 drop by d, and so does the accumulator seed.
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
-        if (__builtin_amdgcn_ballot_w64(mx[qs] > m_ref[qs] + kGrowLog2) != 0) {
-            const float m_new = mx[qs] > m_ref[qs] + kGrowLog2 ? mx[qs] : m_ref[qs];
-            const float fac = __builtin_amdgcn_exp2f(m_ref[qs] - m_new);
-            m_ref[qs] = m_new;
+        if (__builtin_amdgcn_ballot_w64(mx[qs] > kGrowLog2) != 0) {
+            const float d = mx[qs] > kGrowLog2 ? mx[qs] : 0.0f;
+            const float fac = __builtin_amdgcn_exp2f(-d);
             l_run[qs] *= fac;
 #pragma unroll
             for (int t = 0; t < TS; ++t)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) oacc[qs][t][v] *= fac;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                s_next[qs][0][v] -= d;
+                s_next[qs][1][v] -= d;
+                negm[qs][v] -= d;
+            }
         }
     }
 }
@@ -283,10 +288,13 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // Q is in registers: from here on vmcnt counts tile loads only
 
     f32x16 oacc[QS][HD / 32];
-    float m_ref[QS], l_run[QS];
+    // negm = minus the softmax reference of the lane's query row (log2 units), replicated over a 16-register
+    // block so that it can seed the score accumulators: the MFMAs then deliver s - m_ref and no subtraction is
+    // left in the exp path
+    f32x16 negm[QS];
+    float l_run[QS];
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
-        m_ref[qs] = 0.0f;
         l_run[qs] = 0.0f;
 #pragma unroll
         for (int t = 0; t < HD / 32; ++t)
@@ -325,7 +333,13 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         for (int v = 0; v < 16; ++v) { s_a[qs][0][v] = 0.0f; s_a[qs][1][v] = 0.0f; }
         scores_tile<HD>(sk, qf[qs], s_a[qs], lane);
         if (NT == 1 && ragged) mask_scores(s_a[qs], last_valid, lane);
-        m_ref[qs] = tile_row_max(s_a[qs]);      // exact first reference: every row has at least one finite score
+        const float m0 = tile_row_max(s_a[qs]);      // exact first reference: every row has at least one finite score
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            s_a[qs][0][v] -= m0;
+            s_a[qs][1][v] -= m0;
+            negm[qs][v] = -m0;
+        }
     }
     bf16x8 kw[KWIN][2];
     preload_k<HD>(sk + TILE_BYTES, kw, lane);      // K(1) for step 0
@@ -344,7 +358,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         issue(vbase, sv_addr, j + 2, v_fill);                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         pipe_step<HD, QS>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,  \
-                          SCUR, SNEXT, oacc, m_ref, l_run, lane, ragged && j + 2 == NT, last_valid);            \
+                          SCUR, SNEXT, oacc, negm, l_run, lane, ragged && j + 2 == NT, last_valid);            \
         vs_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
