@@ -64,7 +64,7 @@ __device__ __forceinline__ void compute_stage(const char* sa, const char* sb, f3
             for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < 4; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0);
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ni], af[mi], acc[mi][ni], 0, 0, 0);
         }
     } else {
         // 2 x 64 e4m3: a lane supplies 32 consecutive bytes of K (two 16-byte chunks).  The same
@@ -91,7 +91,7 @@ __device__ __forceinline__ void compute_stage(const char* sa, const char* sb, f3
 #pragma unroll
                 for (int ni = 0; ni < 4; ++ni)
                     acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                        af[mi], bfr[ni], acc[mi][ni], 0 /*A: e4m3*/, 0 /*B: e4m3*/, 0, 0x7f7f7f7f /*2^0*/, 0,
+                        bfr[ni], af[mi], acc[mi][ni], 0 /*A: e4m3*/, 0 /*B: e4m3*/, 0, 0x7f7f7f7f /*2^0*/, 0,
                         0x7f7f7f7f);
         }
     }
@@ -111,101 +111,115 @@ __device__ __forceinline__ void issue_loads(const char* abase, const char* wbase
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
 
-// ---- epilogue shared by both pipelines
+// ---- epilogue shared by both pipelines.
+// The MFMAs are issued with the W fragment as the first operand, so an accumulator block holds C TRANSPOSED:
+// element v of block (mi, ni) is output row (token) lane % 32 and output column 8 (v / 4) + 4 (lane / 32) + v % 4 of
+// its 32x32 block.  A lane therefore owns ONE output row per mi and groups of FOUR consecutive columns, and every
+// global access of the epilogue (C, residual, gate, scales, rotary tables) is an 8- or 16-byte vector access.
+// N is a multiple of 8 (host-checked), so a group of four columns is either entirely inside or entirely outside.
+__device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) {
+    return make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+}
+
 template <int EPI, bool FP8>
 __device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4], int m0, int n0, int wm, int wn,
                                          int lane) {
-    // ---- epilogue: accumulator (mi, ni, v) is row 8*(v/4) + 4*(lane/32) + v%4, column lane%32 of its 32x32 block
     const int r32 = lane & 31, kh = lane >> 5;
-    const int row_base = m0 + wm * 128 + 4 * kh;
+    const int row_base = m0 + wm * 128 + r32;
     if (EPI == CDM_EPI_SWIGLU) {
-        const int col_base = n0 + wn * 64 + r32;      // wave's 128 tile columns = [gate 64 | up 64]
+        const int col_base = n0 + wn * 64 + 4 * kh;      // wave's 128 tile columns = [gate 64 | up 64]
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+        for (int mi = 0; mi < 4; ++mi) {
+            const int row = row_base + mi * 32;
+            if (row >= p.M) continue;
+            const float sr = FP8 ? p.sa[row] : 1.0f;
+            bf16_t* crow = p.C + (int64_t)row * p.ldc;
 #pragma unroll
-            for (int nj = 0; nj < 2; ++nj) {
-                const int col = col_base + nj * 32;
-                if (col >= p.N) continue;
-                float sg = 1.0f, su = 1.0f;
-                if (FP8) { sg = p.sw[col]; su = p.sw2[col]; }
+            for (int nj = 0; nj < 2; ++nj)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
-                    if (row < p.M) {
-                        float g = acc[mi][nj][v], u = acc[mi][nj + 2][v];
-                        if (FP8) { const float sr = p.sa[row]; g *= sr * sg; u *= sr * su; }
-                        p.C[(int64_t)row * p.ldc + col] = __builtin_bit_cast(bf16_t, (__bf16)(silu_f(g) * u));
+                for (int g = 0; g < 4; ++g) {
+                    const int col = col_base + nj * 32 + 8 * g;
+                    if (col >= p.N) continue;
+                    float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
+                    if (FP8) {
+                        const float4 a = *reinterpret_cast<const float4*>(p.sw + col);
+                        const float4 b = *reinterpret_cast<const float4*>(p.sw2 + col);
+                        sg[0] = a.x * sr; sg[1] = a.y * sr; sg[2] = a.z * sr; sg[3] = a.w * sr;
+                        su[0] = b.x * sr; su[1] = b.y * sr; su[2] = b.z * sr; su[3] = b.w * sr;
                     }
+                    float o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        o[e] = silu_f(acc[mi][nj][4 * g + e] * sg[e]) * (acc[mi][nj + 2][4 * g + e] * su[e]);
+                    *reinterpret_cast<uint2*>(crow + col) = pack4_bf16(o[0], o[1], o[2], o[3]);
                 }
-            }
+        }
         return;
     }
-    const int col_base = n0 + wn * 128 + r32;
-    if (FP8) {      // rank-1 dequantisation scale on the fp32 accumulators
-        float sc[4];
+    const int col_base = n0 + wn * 128 + 4 * kh;
+    const bool rope = EPI == CDM_EPI_ROPE_QK && n0 + wn * 128 < p.rope_cols;   // wave-uniform: whole heads of Q or K
+    const int half = p.head_dim >> 1;
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) { const int col = col_base + ni * 32; sc[ni] = col < p.N ? p.sw[col] : 0.0f; }
+    for (int mi = 0; mi < 4; ++mi) {
+        const int row = row_base + mi * 32;
+        if (row >= p.M) continue;
+        if (FP8) {      // rank-1 dequantisation scale on the fp32 accumulators
+            const float sr = p.sa[row];
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+            for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
-                const float sr = p.sa[row < p.M ? row : p.M - 1];
+                for (int g = 0; g < 4; ++g) {
+                    const int col = col_base + ni * 32 + 8 * g;
+                    const float4 w4 = col < p.N ? *reinterpret_cast<const float4*>(p.sw + col) : make_float4(0, 0, 0, 0);
+                    acc[mi][ni][4 * g + 0] *= sr * w4.x;
+                    acc[mi][ni][4 * g + 1] *= sr * w4.y;
+                    acc[mi][ni][4 * g + 2] *= sr * w4.z;
+                    acc[mi][ni][4 * g + 3] *= sr * w4.w;
+                }
+        }
+        if (EPI == CDM_EPI_ROPE_QK && rope) {
+            // rotate-half pairs (i, i + head_dim/2).  head_dim 128: blocks (nj, nj + 2), pair index 32 nj + ...;
+            // head_dim 64: two heads per wave, blocks (nj, nj + 1) with nj even, pair index inside the block
+            const float* cr = p.cos + (int64_t)row * half;
+            const float* sr_ = p.sin + (int64_t)row * half;
 #pragma unroll
-                for (int ni = 0; ni < 4; ++ni) acc[mi][ni][v] *= sr * sc[ni];
-            }
-    }
-    if (EPI == CDM_EPI_ROPE_QK) {
-        if (n0 + wn * 128 < p.rope_cols) {     // wave-uniform: this wave's 128 columns are whole heads of Q or K
-            const int half = p.head_dim >> 1;
+            for (int nj = 0; nj < 2; ++nj)
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
+                for (int g = 0; g < 4; ++g) {
+                    const int lo = p.head_dim == 128 ? nj : 2 * nj, hi = p.head_dim == 128 ? nj + 2 : 2 * nj + 1;
+                    const int i = (p.head_dim == 128 ? nj * 32 : 0) + 8 * g + 4 * kh;
+                    const float4 c4 = *reinterpret_cast<const float4*>(cr + i);
+                    const float4 s4 = *reinterpret_cast<const float4*>(sr_ + i);
+                    const float c[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
-                    const int rr = row < p.M ? row : p.M - 1;
-                    if (p.head_dim == 128) {
-#pragma unroll
-                        for (int nj = 0; nj < 2; ++nj) {
-                            const int i = nj * 32 + r32;
-                            const float c = p.cos[(int64_t)rr * half + i], s = p.sin[(int64_t)rr * half + i];
-                            const float x1 = acc[mi][nj][v], x2 = acc[mi][nj + 2][v];
-                            acc[mi][nj][v] = x1 * c - x2 * s;
-                            acc[mi][nj + 2][v] = x2 * c + x1 * s;
-                        }
-                    } else {   // head_dim 64: two heads per wave, pairs are adjacent 32-column blocks
-                        const float c = p.cos[(int64_t)rr * half + r32], s = p.sin[(int64_t)rr * half + r32];
-#pragma unroll
-                        for (int nj = 0; nj < 4; nj += 2) {
-                            const float x1 = acc[mi][nj][v], x2 = acc[mi][nj + 1][v];
-                            acc[mi][nj][v] = x1 * c - x2 * s;
-                            acc[mi][nj + 1][v] = x2 * c + x1 * s;
-                        }
+                    for (int e = 0; e < 4; ++e) {
+                        const float x1 = acc[mi][lo][4 * g + e], x2 = acc[mi][hi][4 * g + e];
+                        acc[mi][lo][4 * g + e] = x1 * c[e] - x2 * sn[e];
+                        acc[mi][hi][4 * g + e] = x2 * c[e] + x1 * sn[e];
                     }
                 }
         }
-    }
+        bf16_t* crow = p.C + (int64_t)row * p.ldc;
+        const bf16_t* rrow = EPI == CDM_EPI_GATE_RESIDUAL ? p.R + (int64_t)row * p.ldr : nullptr;
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+        for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) {
-            const int col = col_base + ni * 32;
-            if (col >= p.N) continue;
-            float gt = 1.0f;
-            if (EPI == CDM_EPI_GATE_RESIDUAL && p.gate) gt = p.gate[col];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = row_base + mi * 32 + 8 * (v >> 2) + (v & 3);
-                if (row < p.M) {
-                    float val = acc[mi][ni][v];
-                    if (EPI == CDM_EPI_GATE_RESIDUAL) {
-                        const float res = bf16_bits_to_f32(p.R[(int64_t)row * p.ldr + col]);
-                        val = res + gt * val;
-                    }
-                    p.C[(int64_t)row * p.ldc + col] = __builtin_bit_cast(bf16_t, (__bf16)val);
+            for (int g = 0; g < 4; ++g) {
+                const int col = col_base + ni * 32 + 8 * g;
+                if (col >= p.N) continue;
+                float o[4] = {acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]};
+                if (EPI == CDM_EPI_GATE_RESIDUAL) {
+                    const uint2 r2 = *reinterpret_cast<const uint2*>(rrow + col);
+                    float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
+                    if (p.gate) g4 = *reinterpret_cast<const float4*>(p.gate + col);
+                    o[0] = bf16lo(r2.x) + g4.x * o[0];
+                    o[1] = bf16hi(r2.x) + g4.y * o[1];
+                    o[2] = bf16lo(r2.y) + g4.z * o[2];
+                    o[3] = bf16hi(r2.y) + g4.w * o[3];
                 }
+                *reinterpret_cast<uint2*>(crow + col) = pack4_bf16(o[0], o[1], o[2], o[3]);
             }
-        }
+    }
 }
 
 template <int EPI, bool FP8>
@@ -417,11 +431,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto mfma = [&](const Frags<FP8>& f, int i) {
         const int mi = i >> 2, ni = i & 3;
         if constexpr (FP8)
-            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[mi], f.b[ni], acc[mi][ni], 0 /*A: e4m3*/,
+            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[ni], f.a[mi], acc[mi][ni], 0 /*A: e4m3*/,
                                                                           0 /*B: e4m3*/, 0, 0x7f7f7f7f /*2^0*/, 0,
                                                                           0x7f7f7f7f);
         else
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[mi], f.b[ni], acc[mi][ni], 0, 0, 0);
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[ni], f.a[mi], acc[mi][ni], 0, 0, 0);
     };
     // prologue: granules 0..3 (tiles 0 and 1)
 #pragma unroll
@@ -493,12 +507,18 @@ int32_t validate(const char* who, int esize, const void* A, int64_t lda, const v
     CDM_REQUIRE(cdm_aligned16(A) && cdm_aligned16(W) && cdm_aligned16(C) && (lda * esize) % 16 == 0 &&
                     (ldw * esize) % 16 == 0,
                 CDM_ERR_BAD_ALIGN, "%s: pointers/strides must be 16-byte aligned", who);
+    CDM_REQUIRE(ldc % 8 == 0, CDM_ERR_BAD_ALIGN, "%s: ldc=%lld must be a multiple of 8 elements", who, (long long)ldc);
     if (epi == CDM_EPI_SWIGLU)
         CDM_REQUIRE(W2 && cdm_aligned16(W2), CDM_ERR_BAD_ARG, "%s: SWIGLU needs an aligned W2 (up_proj)", who);
     if (epi == CDM_EPI_GATE_RESIDUAL)
+    {
         CDM_REQUIRE(R && ldr >= N, CDM_ERR_BAD_ARG, "%s: GATE_RESIDUAL needs R with ldr >= N", who);
+        CDM_REQUIRE(cdm_aligned16(R) && ldr % 8 == 0, CDM_ERR_BAD_ALIGN,
+                    "%s: residual pointer / row stride must be 16-byte aligned", who);
+    }
     if (epi == CDM_EPI_ROPE_QK) {
         CDM_REQUIRE(cos && sin, CDM_ERR_BAD_ARG, "%s: ROPE_QK needs cos/sin tables", who);
+        CDM_REQUIRE(cdm_aligned16(cos) && cdm_aligned16(sin), CDM_ERR_BAD_ALIGN, "%s: cos/sin must be 16-byte aligned", who);
         CDM_REQUIRE(head_dim == 64 || head_dim == 128, CDM_ERR_BAD_SHAPE, "%s: head_dim=%d must be 64 or 128", who,
                     head_dim);
         CDM_REQUIRE(rope_cols >= 0 && rope_cols <= N && rope_cols % 256 == 0, CDM_ERR_BAD_SHAPE,
@@ -538,6 +558,7 @@ extern "C" int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int6
     int32_t rc = validate("gemm_bf16", 2, A, lda, W, ldw, W2, C, ldc, M, N, K, epilogue, R, ldr, cos, sin, rope_cols,
                           head_dim);
     if (rc) return rc;
+    CDM_REQUIRE(cdm_aligned16(gate), CDM_ERR_BAD_ALIGN, "gemm_bf16: gate must be 16-byte aligned");
     if ((rc = cdm_require_device())) return rc;
     if (M == 0) return CDM_OK;
     GemmParams p{};
@@ -560,6 +581,8 @@ extern "C" int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, co
     if (rc) return rc;
     CDM_REQUIRE(sa && sw, CDM_ERR_BAD_ARG, "gemm_fp8: null scale pointer");
     if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(sw2, CDM_ERR_BAD_ARG, "gemm_fp8: SWIGLU needs sw2");
+    CDM_REQUIRE(cdm_aligned16(gate) && cdm_aligned16(sw) && cdm_aligned16(sw2), CDM_ERR_BAD_ALIGN,
+                "gemm_fp8: gate and weight-scale vectors must be 16-byte aligned");
     if ((rc = cdm_require_device())) return rc;
     if (M == 0) return CDM_OK;
     GemmParams p{};

@@ -96,7 +96,8 @@ int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, float* s, int64
  *   CDM_EPI_ROPE_QK:       cos, sin: [M, head_dim/2] fp32; columns [0, rope_cols) are rotated
  *                          per head (pairs (i, i + head_dim/2)); head_dim in {64, 128};
  *                          rope_cols % 256 == 0
- * K % 128 == 0; M, N >= 1 arbitrary (N % 8 == 0).
+ * K % 128 == 0; M, N >= 1 arbitrary (N % 8 == 0); ldc and ldr multiples of 8 elements (every output and residual
+ * row starts on a 16-byte boundary: the epilogue moves groups of four columns per lane).
  */
 int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2,
                       void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epilogue,
