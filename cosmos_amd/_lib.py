@@ -21,6 +21,12 @@ EPI_NONE, EPI_SWIGLU, EPI_GATE_RESIDUAL, EPI_ROPE_QK = 0, 1, 2, 3
 _P, _I64, _I32, _F32 = C.c_void_p, C.c_int64, C.c_int32, C.c_float
 
 # name -> (restype, argtypes); mirrors include/cosmos_dm.h one to one
+class QkNorm(C.Structure):
+    """Mirror of ``cdm_qk_norm``: device weight tables [n_seg, head_dim] fp32, host segment ends, eps."""
+    _fields_ = [("q_weight", C.c_void_p), ("k_weight", C.c_void_p), ("seg_end", C.POINTER(C.c_int64)),
+                ("n_seg", C.c_int32), ("eps", C.c_float)]
+
+
 SIGNATURES = {
     "cdm_version": (_I32, []),
     "cdm_last_error": (C.c_char_p, []),
@@ -35,9 +41,9 @@ SIGNATURES = {
                             _P, _I64, _I32, _P]),
     "cdm_mrope_qk_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I32, _I32, _P]),
     "cdm_attn_workspace_bytes": (_I64, [_I64, _I32, _I32]),
-    "cdm_attn_fwd_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _I64, _P]),
-    "cdm_attn_pack_kv_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P]),
-    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _P]),
+    "cdm_attn_fwd_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _I64, _P, _P]),
+    "cdm_attn_pack_kv_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _P]),
+    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _P]),
     "cdm_grouped_gemm_bf16": (_I32, [_P, _I64, C.POINTER(_P), _I64, C.POINTER(_P), _P, _I64, C.POINTER(_I64),
                                      C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P, _P, _I64,
                                      _I32, _P]),

@@ -22,6 +22,7 @@ class DMConfig:
     rope_layout: str = "chunked"
     eps: float = 1e-6
     fp8: bool = False
+    qk_norm: bool = False                    # per-head RMSNorm of Q and K ahead of the rotation
     seed: int = 1234
 
     @property

@@ -215,12 +215,28 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
     }
 }
 
+// Per-head RMSNorm of Q / K ahead of the rotation: y = x * rsqrt(mean(x^2) + eps) * w[segment], in fp32.
+// Segments are contiguous token ranges [seg_end[i-1], seg_end[i]) with their own weight row (MoT branches).
+struct QkNormDev {
+    const float* w;        // [n_seg, HD] or null = no normalisation
+    int seg_end[8];
+    int n_seg;
+    float eps;
+    __device__ __forceinline__ const float* row(int token, int hd) const {
+        int sidx = 0;
+#pragma unroll
+        for (int i = 0; i < 7; ++i) sidx += (i < n_seg - 1 && token >= seg_end[i]) ? 1 : 0;
+        return w + sidx * hd;
+    }
+};
+
 struct PackedParams {
     const bf16_t* q; int64_t ldq;
     const char* kp;              // [n_heads][n_tiles][tile bytes]
     const char* vp;
     bf16_t* o; int64_t ldo;
     const float* cos; const float* sin;   // optional rotary tables [n_tokens, HD/2] applied to Q at load
+    QkNormDev qn;                          // optional per-head RMSNorm of Q, applied before the rotation
     int n_tokens, n_heads;
     float scale_log2e;
 };
@@ -257,10 +273,31 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qp + 16 * ks);
+        // per-head RMSNorm: the lane holds 8 channels per k-step, its partner (lane ^ 32) the other 8
+        float rnorm = 1.0f;
+        const float* nw = nullptr;
+        if (p.qn.w != nullptr) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint32_t w[4] = {raw[ks].x, raw[ks].y, raw[ks].z, raw[ks].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { const float a = bf16lo(w[j]), b = bf16hi(w[j]); ss += a * a + b * b; }
+            }
+            ss += __shfl_xor(ss, 32, 64);
+            rnorm = rsqrtf(ss * (1.0f / HD) + p.qn.eps);
+            nw = p.qn.row(qrow, HD) + 8 * kh;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS / 2; ++ks) {
             const uint32_t w1[4] = {raw[ks].x, raw[ks].y, raw[ks].z, raw[ks].w};
             const uint32_t w2[4] = {raw[ks + KS / 2].x, raw[ks + KS / 2].y, raw[ks + KS / 2].z, raw[ks + KS / 2].w};
+            float n1[8], n2[8];      // norm factors of the channels of k-step ks and of its rotary partners
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                n1[e] = nw ? rnorm * nw[16 * ks + e] : 1.0f;
+                n2[e] = nw ? rnorm * nw[16 * (ks + KS / 2) + e] : 1.0f;
+            }
             float c[8], sn[8];
             if (p.cos != nullptr) {
                 const float4* cp = reinterpret_cast<const float4*>(p.cos + (int64_t)qrow * (HD / 2) + 16 * ks + 8 * kh);
@@ -275,7 +312,8 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             uint32_t o1[4], o2[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float a0 = bf16lo(w1[j]), a1 = bf16hi(w1[j]), b0 = bf16lo(w2[j]), b1 = bf16hi(w2[j]);
+                const float a0 = bf16lo(w1[j]) * n1[2 * j], a1 = bf16hi(w1[j]) * n1[2 * j + 1];
+                const float b0 = bf16lo(w2[j]) * n2[2 * j], b1 = bf16hi(w2[j]) * n2[2 * j + 1];
                 o1[j] = pack_bf16x2((a0 * c[2 * j] - b0 * sn[2 * j]) * p.scale_log2e,
                                     (a1 * c[2 * j + 1] - b1 * sn[2 * j + 1]) * p.scale_log2e);
                 o2[j] = pack_bf16x2((b0 * c[2 * j] + a0 * sn[2 * j]) * p.scale_log2e,
@@ -396,8 +434,8 @@ template <int HD>
 __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__ k, int64_t ldk,
                                                       const bf16_t* __restrict__ v, int64_t ldv,
                                                       const float* __restrict__ cos, const float* __restrict__ sin,
-                                                      char* __restrict__ kp, char* __restrict__ vp, int n_tokens,
-                                                      int n_tiles) {
+                                                      const QkNormDev kn, char* __restrict__ kp, char* __restrict__ vp,
+                                                      int n_tokens, int n_tiles) {
     __shared__ bf16_t tile[64][HD + 2];
     constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
     constexpr int HALF = HD / 2;
@@ -417,17 +455,38 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
             k2 = *reinterpret_cast<const uint4*>(kr + HALF);
             v1 = *reinterpret_cast<const uint4*>(vr);
             v2 = *reinterpret_cast<const uint4*>(vr + HALF);
-            if (cos != nullptr) {
-                const float4* cp = reinterpret_cast<const float4*>(cos + (int64_t)(t0 + r) * HALF + ch * 8);
-                const float4* sp = reinterpret_cast<const float4*>(sin + (int64_t)(t0 + r) * HALF + ch * 8);
-                const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
-                const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-                const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            if (cos != nullptr || kn.w != nullptr) {
+                float c[8], sn[8], n1[8], n2[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { c[e] = 1.0f; sn[e] = 0.0f; n1[e] = 1.0f; n2[e] = 1.0f; }
                 const uint32_t w1[4] = {k1.x, k1.y, k1.z, k1.w}, w2[4] = {k2.x, k2.y, k2.z, k2.w};
+                if (kn.w != nullptr) {
+                    // per-head RMSNorm: the CPR/2 consecutive threads of a token hold its HD channels
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float a0 = bf16lo(w1[j]), a1 = bf16hi(w1[j]), b0 = bf16lo(w2[j]), b1 = bf16hi(w2[j]);
+                        ss += a0 * a0 + a1 * a1 + b0 * b0 + b1 * b1;
+                    }
+#pragma unroll
+                    for (int off = 1; off < CPR / 2; off <<= 1) ss += __shfl_xor(ss, off, 64);
+                    const float rn = rsqrtf(ss * (1.0f / HD) + kn.eps);
+                    const float* nw = kn.row(t0 + r, HD) + ch * 8;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) { n1[e] = rn * nw[e]; n2[e] = rn * nw[HALF + e]; }
+                }
+                if (cos != nullptr) {
+                    const float4* cp = reinterpret_cast<const float4*>(cos + (int64_t)(t0 + r) * HALF + ch * 8);
+                    const float4* sp = reinterpret_cast<const float4*>(sin + (int64_t)(t0 + r) * HALF + ch * 8);
+                    const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+                    c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+                    sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+                }
                 uint32_t o1[4], o2[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float a0 = bf16lo(w1[j]), a1 = bf16hi(w1[j]), b0 = bf16lo(w2[j]), b1 = bf16hi(w2[j]);
+                    const float a0 = bf16lo(w1[j]) * n1[2 * j], a1 = bf16hi(w1[j]) * n1[2 * j + 1];
+                    const float b0 = bf16lo(w2[j]) * n2[2 * j], b1 = bf16hi(w2[j]) * n2[2 * j + 1];
                     o1[j] = pack_bf16x2(a0 * c[2 * j] - b0 * sn[2 * j], a1 * c[2 * j + 1] - b1 * sn[2 * j + 1]);
                     o2[j] = pack_bf16x2(b0 * c[2 * j] + a0 * sn[2 * j], b1 * c[2 * j + 1] + a1 * sn[2 * j + 1]);
                 }
@@ -458,6 +517,28 @@ inline int64_t image_bytes(int64_t n_tokens, int n_heads, int head_dim) {      /
     return pad_tokens(n_tokens) * n_heads * head_dim * 2;
 }
 
+// host view of the optional QK-norm argument -> kernel descriptor (which = 0: q weights, 1: k weights)
+int32_t make_qk_norm(const char* who, const cdm_qk_norm* qn, int which, int64_t n_tokens, QkNormDev* out) {
+    out->w = nullptr; out->n_seg = 0; out->eps = 0.0f;
+    for (int i = 0; i < 8; ++i) out->seg_end[i] = 0;
+    if (qn == nullptr) return CDM_OK;
+    const float* w = which == 0 ? qn->q_weight : qn->k_weight;
+    CDM_REQUIRE(qn->q_weight && qn->k_weight, CDM_ERR_BAD_ARG, "%s: qk_norm needs both weight tables", who);
+    CDM_REQUIRE(qn->n_seg >= 1 && qn->n_seg <= 8 && qn->seg_end, CDM_ERR_BAD_ARG, "%s: qk_norm n_seg=%d must be 1..8", who,
+                qn->n_seg);
+    CDM_REQUIRE(qn->eps > 0.0f, CDM_ERR_BAD_ARG, "%s: qk_norm eps must be positive", who);
+    int64_t prev = 0;
+    for (int i = 0; i < qn->n_seg; ++i) {
+        CDM_REQUIRE(qn->seg_end[i] >= prev, CDM_ERR_BAD_ARG, "%s: qk_norm segment ends must not decrease", who);
+        prev = qn->seg_end[i];
+        out->seg_end[i] = (int)(prev < (1ll << 30) ? prev : (1ll << 30));
+    }
+    CDM_REQUIRE(prev >= n_tokens, CDM_ERR_BAD_ARG, "%s: qk_norm segments cover %lld of %lld tokens", who, (long long)prev,
+                (long long)n_tokens);
+    out->w = w; out->n_seg = qn->n_seg; out->eps = qn->eps;
+    return CDM_OK;
+}
+
 int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, int32_t head_dim, const float* cos,
                           const float* sin) {
     CDM_REQUIRE(n_tokens >= 0 && n_heads > 0, CDM_ERR_BAD_ARG, "%s: bad sizes", who);
@@ -478,10 +559,13 @@ extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, i
 
 extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                                          const float* sin, void* workspace, int64_t workspace_bytes,
-                                         int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream) {
+                                         int64_t n_tokens, int32_t n_heads, int32_t head_dim,
+                                         const cdm_qk_norm* qk_norm, void* stream) {
     CDM_REQUIRE(k && v && workspace, CDM_ERR_BAD_ARG, "attn_pack_kv: null pointer");
     int32_t rc = check_attn_common("attn_pack_kv", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
+    QkNormDev kn;
+    if ((rc = make_qk_norm("attn_pack_kv", qk_norm, 1, n_tokens, &kn))) return rc;
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldk >= d && ldv >= d, CDM_ERR_BAD_ARG, "attn_pack_kv: row stride smaller than n_heads*head_dim");
     CDM_REQUIRE(cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(workspace) && ldk % 8 == 0 && ldv % 8 == 0,
@@ -497,20 +581,23 @@ extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void*
     dim3 grid(n_tiles, n_heads);
     hipStream_t st = (hipStream_t)stream;
     if (head_dim == 128)
-        pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, ws, ws + img,
+        pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, kn, ws, ws + img,
                                                   (int)n_tokens, n_tiles);
     else
-        pack_kv_kernel<64><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, ws, ws + img,
+        pack_kv_kernel<64><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, kn, ws, ws + img,
                                                  (int)n_tokens, n_tiles);
     return cdm_check_launch("attn_pack_kv");
 }
 
 extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
                                             const void* workspace, void* o, int64_t ldo, int64_t n_tokens,
-                                            int32_t n_heads, int32_t head_dim, void* stream) {
+                                            int32_t n_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
+                                            void* stream) {
     CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
     int32_t rc = check_attn_common("attn_fwd_packed", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
+    QkNormDev qn;
+    if ((rc = make_qk_norm("attn_fwd_packed", qk_norm, 0, n_tokens, &qn))) return rc;
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldq >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd_packed: row stride smaller than n_heads*head_dim");
     CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(workspace) && cdm_aligned16(o) && ldq % 8 == 0 && ldo % 4 == 0,
@@ -523,6 +610,7 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     p.kp = (const char*)workspace; p.vp = (const char*)workspace + img;
     p.o = (bf16_t*)o; p.ldo = ldo;
     p.cos = cos; p.sin = sin;
+    p.qn = qn;
     p.n_tokens = (int)n_tokens; p.n_heads = n_heads;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
     dim3 grid((unsigned)((n_tokens + BMQ - 1) / BMQ), n_heads);
@@ -541,10 +629,14 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
 extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                                      int64_t ldv, const float* cos, const float* sin, void* o, int64_t ldo,
                                      int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* workspace,
-                                     int64_t workspace_bytes, void* stream) {
+                                     int64_t workspace_bytes, const cdm_qk_norm* qk_norm, void* stream) {
     CDM_REQUIRE(q && k && v && o, CDM_ERR_BAD_ARG, "attn_fwd: null pointer");
     int32_t rc = check_attn_common("attn_fwd", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
+    {
+        QkNormDev tmp;
+        if ((rc = make_qk_norm("attn_fwd", qk_norm, 0, n_tokens, &tmp))) return rc;
+    }
     if (n_tokens == 0) return CDM_OK;
     const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim);
     CDM_REQUIRE(workspace && cdm_aligned16(workspace) && workspace_bytes >= need, CDM_ERR_BAD_ARG,
@@ -556,7 +648,7 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
                     ldk % 8 == 0 && ldv % 8 == 0 && ldo % 4 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
     if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_heads, head_dim,
-                                    stream)))
+                                    qk_norm, stream)))
         return rc;
-    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, head_dim, stream);
+    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, head_dim, qk_norm, stream);
 }

@@ -100,6 +100,9 @@ class DMAttnProcessor:
 
         wsb = ws.attn_ws if ws is not None else None
         q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
+        qkn = attn.qk_norm_args(modality_segments)
+        if qkn is not None and self.rope != "in_attention":
+            raise NotImplementedError("QK-RMSNorm precedes the rotation: it needs rope='in_attention'")
         if self.rope == "gemm_epilogue":
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
                          rope_cols=2 * d, head_dim=attn.head_dim)
@@ -110,7 +113,8 @@ class DMAttnProcessor:
                 ops.mrope_qk_(q, k, cos, sin, attn.n_heads, attn.head_dim)
                 ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb)
             else:     # in registers, inside the attention kernels
-                ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin)
+                ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin,
+                              qk_norm=qkn)
         if attn.fp8:
             oq, so = ops.quant_rows(o)
         else:
@@ -133,12 +137,21 @@ class DMAttention(nn.Module):
     """Attention module of one MoT layer: per-branch projections around one shared attention."""
 
     def __init__(self, d_model: int, n_heads: int, head_dim: int, n_branches: int = 1, fp8: bool = False,
-                 processor: Optional[DMAttnProcessor] = None, device=None, dtype=torch.bfloat16):
+                 processor: Optional[DMAttnProcessor] = None, device=None, dtype=torch.bfloat16,
+                 qk_norm: bool = False, eps: float = 1e-6):
         super().__init__()
         if n_heads * head_dim != d_model:
             raise ValueError("n_heads * head_dim must equal d_model")
         self.d_model, self.n_heads, self.head_dim, self.n_branches, self.fp8 = d_model, n_heads, head_dim, n_branches, fp8
         kw = dict(device=device, dtype=dtype)
+        # per-head QK-RMSNorm weights, one row per branch (norm_q / norm_added_q and norm_k / norm_added_k of the
+        # reference's attention layer); fp32 because the kernels normalise in fp32
+        self.qk_norm, self.qk_eps = qk_norm, eps
+        if qk_norm:
+            self.norm_q_weight = nn.Parameter(torch.ones(n_branches, head_dim, device=device, dtype=torch.float32),
+                                              requires_grad=False)
+            self.norm_k_weight = nn.Parameter(torch.ones(n_branches, head_dim, device=device, dtype=torch.float32),
+                                              requires_grad=False)
         self.qkv_weight = nn.ParameterList([nn.Parameter(torch.empty(3 * d_model, d_model, **kw), requires_grad=False)
                                             for _ in range(n_branches)])
         self.out_weight = nn.ParameterList([nn.Parameter(torch.empty(d_model, d_model, **kw), requires_grad=False)
@@ -156,6 +169,18 @@ class DMAttention(nn.Module):
 
     def _weights(self, which: str):
         return self.qkv_weight if which == "qkv" else self.out_weight
+
+    def qk_norm_args(self, segments: Sequence[Segment]):
+        """(q_weight, k_weight, seg_ends, eps) for ``ops.attention``: one weight row per token segment."""
+        if not self.qk_norm:
+            return None
+        branches = [b for (_, _, b, _) in segments]
+        ends = [s0 + ln for (s0, ln, _, _) in segments]
+        qw, kw = self.norm_q_weight.data, self.norm_k_weight.data
+        if branches != list(range(self.n_branches)):
+            idx = torch.tensor(branches, device=qw.device)
+            qw, kw = qw.index_select(0, idx).contiguous(), kw.index_select(0, idx).contiguous()
+        return qw, kw, ends, self.qk_eps
 
     def _linear(self, a: torch.Tensor, sa: Optional[torch.Tensor], which: str, segments: Sequence[Segment], *,
                 out: torch.Tensor, epilogue: str, residual=None, gates=None, cos=None, sin=None, rope_cols=0,
@@ -195,11 +220,12 @@ class DMBlock(nn.Module):
     """One Mixture-of-Transformers layer (generator side)."""
 
     def __init__(self, d_model: int, n_heads: int, head_dim: int, hidden: int, n_branches: int = 1,
-                 eps: float = 1e-6, fp8: bool = False, device=None, dtype=torch.bfloat16):
+                 eps: float = 1e-6, fp8: bool = False, device=None, dtype=torch.bfloat16, qk_norm: bool = False):
         super().__init__()
         kw = dict(device=device, dtype=dtype)
         self.d_model, self.hidden, self.eps, self.fp8, self.n_branches = d_model, hidden, eps, fp8, n_branches
-        self.attn = DMAttention(d_model, n_heads, head_dim, n_branches, fp8, device=device, dtype=dtype)
+        self.attn = DMAttention(d_model, n_heads, head_dim, n_branches, fp8, device=device, dtype=dtype,
+                                qk_norm=qk_norm, eps=eps)
         P = lambda *shape: nn.Parameter(torch.empty(*shape, **kw), requires_grad=False)
         self.norm1_weight = nn.ParameterList([P(d_model) for _ in range(n_branches)])
         self.norm2_weight = nn.ParameterList([P(d_model) for _ in range(n_branches)])
@@ -310,7 +336,7 @@ class DMStack(nn.Module):
         self.cfg = cfg
         self.time_embedder = TimestepEmbedder(cfg.d_model, device=device)
         self.blocks = nn.ModuleList([DMBlock(cfg.d_model, cfg.n_heads, cfg.head_dim, cfg.hidden, cfg.n_branches,
-                                             cfg.eps, cfg.fp8, device=device, dtype=dtype)
+                                             cfg.eps, cfg.fp8, device=device, dtype=dtype, qk_norm=cfg.qk_norm)
                                      for _ in range(cfg.n_blocks)])
         self._rot = None
         self._ws: Optional[Workspace] = None

@@ -205,9 +205,12 @@ def attn_workspace_bytes(n_tokens: int, n_heads: int, head_dim: int) -> int:
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
               out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-              cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+              cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+              qk_norm=None) -> torch.Tensor:
     """Full non-causal attention; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free).
-    With cos/sin ([n, head_dim/2] fp32) rotate-half mRoPE is applied to Q and K inside the kernels."""
+    With cos/sin ([n, head_dim/2] fp32) rotate-half mRoPE is applied to Q and K inside the kernels.
+    ``qk_norm`` = (q_weight, k_weight, seg_ends, eps) switches on the per-head RMSNorm of Q and K ahead of the
+    rotation: weights [n_seg, head_dim] fp32 on the device, ``seg_ends`` the exclusive end token of each segment."""
     lib = _lib.load()
     n = q.shape[0]
     d = n_heads * head_dim
@@ -222,18 +225,26 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     qp, kp, vp = _chk(q, "q", torch.bfloat16, 2), _chk(k, "k", torch.bfloat16, 2), _chk(v, "v", torch.bfloat16, 2)
     op, wp = _chk(out, "out", torch.bfloat16, 2), _chk(workspace, "workspace", torch.uint8, 1)
     cp, sp = _f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half)
+    qn = None
+    if qk_norm is not None:
+        qw, kw, seg_ends, eps = qk_norm
+        seg_ends = [int(e) for e in seg_ends]
+        ends = (C.c_int64 * len(seg_ends))(*seg_ends)
+        qn_struct = _lib.QkNorm(_f32vec(qw, "qk_norm q_weight", len(seg_ends) * head_dim),
+                                _f32vec(kw, "qk_norm k_weight", len(seg_ends) * head_dim), ends, len(seg_ends), float(eps))
+        qn = C.addressof(qn_struct)        # qn_struct and ends stay alive until the calls below have returned
     if _ATTN_TIMER is None:
         rc = lib.cdm_attn_fwd_bf16(qp, q.stride(0), kp, k.stride(0), vp, v.stride(0), cp, sp, op, out.stride(0), n,
-                                   n_heads, head_dim, wp, workspace.numel(), _stream())
+                                   n_heads, head_dim, wp, workspace.numel(), qn, _stream())
         _lib.check(rc, "cdm_attn_fwd_bf16")
         return out
     # timed form: the same two stages, with HIP events around the attention kernel alone
     rc = lib.cdm_attn_pack_kv_bf16(kp, k.stride(0), vp, v.stride(0), cp, sp, wp, workspace.numel(), n, n_heads,
-                                   head_dim, _stream())
+                                   head_dim, qn, _stream())
     _lib.check(rc, "cdm_attn_pack_kv_bf16")
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    rc = lib.cdm_attn_fwd_packed_bf16(qp, q.stride(0), cp, sp, wp, op, out.stride(0), n, n_heads, head_dim, _stream())
+    rc = lib.cdm_attn_fwd_packed_bf16(qp, q.stride(0), cp, sp, wp, op, out.stride(0), n, n_heads, head_dim, qn, _stream())
     e1.record()
     _lib.check(rc, "cdm_attn_fwd_packed_bf16")
     _ATTN_TIMER.append((e0, e1))

@@ -129,6 +129,25 @@ int32_t cdm_mrope_qk_bf16(void* q, int64_t ldq, void* k, int64_t ldk, const floa
                           int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* stream);
 
 /*
+ * Optional per-head QK-RMSNorm, applied to Q and K in fp32 ahead of the rotation inside the attention entry
+ * points - replaces the q_norm / k_norm modules of the attention layer (parameters norm_q / norm_k of the AR
+ * branch and norm_added_q / norm_added_k of the DM branch, transformers
+ * models/cosmos3_omni/modeling_cosmos3_omni.py:45-46; application order norm -> RoPE:
+ * models/qwen3_vl/modeling_qwen3_vl.py:463-466,479-481; RMSNorm :400-405):
+ *   y = x * rsqrt(mean_over_head_dim(x^2) + eps) * weight.
+ * Tokens form n_seg (1..8) contiguous segments, segment i = [seg_end[i-1], seg_end[i]) with seg_end[-1] = 0 and
+ * seg_end[n_seg-1] >= n_tokens; segment i uses row i of the weight tables (one row per MoT branch).
+ * The struct itself and seg_end are HOST memory, read during the call; the weight tables are device memory.
+ */
+typedef struct cdm_qk_norm {
+    const float* q_weight;    /* device, [n_seg, head_dim] fp32 */
+    const float* k_weight;    /* device, [n_seg, head_dim] fp32 */
+    const int64_t* seg_end;   /* host, [n_seg] */
+    int32_t n_seg;
+    float eps;
+} cdm_qk_norm;
+
+/*
  * Shared full (non-causal) self-attention over the joint sequence, with rotate-half mRoPE applied in
  * registers to Q and K on the way in - replaces the attention processor's apply_rotary_pos_emb +
  * scaled_dot_product_attention (README.md:74; eager form transformers
@@ -136,6 +155,7 @@ int32_t cdm_mrope_qk_bf16(void* q, int64_t ldq, void* k, int64_t ldk, const floa
  *   O = softmax(rope(Q) rope(K)^T / sqrt(head_dim)) V per head, no mask.
  *   q, k, v: [n_tokens, n_heads, head_dim] with row strides ldq, ldk, ldv; o: [n_tokens, n_heads*head_dim] (ldo).
  *   cos, sin: [n_tokens, head_dim/2] fp32 rotary tables, or both null when Q and K are already rotated.
+ *   qk_norm: null, or the per-head RMSNorm of Q and K described above.
  *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds K and V re-laid
  *   out as 64-key tile images); its contents are undefined afterwards.
  * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
@@ -143,7 +163,8 @@ int32_t cdm_mrope_qk_bf16(void* q, int64_t ldq, void* k, int64_t ldk, const floa
 int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim);
 int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
                           const float* cos, const float* sin, void* o, int64_t ldo, int64_t n_tokens,
-                          int32_t n_heads, int32_t head_dim, void* workspace, int64_t workspace_bytes, void* stream);
+                          int32_t n_heads, int32_t head_dim, void* workspace, int64_t workspace_bytes,
+                          const cdm_qk_norm* qk_norm, void* stream);
 
 /*
  * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first K (rotated
@@ -153,10 +174,10 @@ int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk
  */
 int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                               const float* sin, void* workspace, int64_t workspace_bytes, int64_t n_tokens,
-                              int32_t n_heads, int32_t head_dim, void* stream);
+                              int32_t n_heads, int32_t head_dim, const cdm_qk_norm* qk_norm, void* stream);
 int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
                                  const void* workspace, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
-                                 int32_t head_dim, void* stream);
+                                 int32_t head_dim, const cdm_qk_norm* qk_norm, void* stream);
 
 /*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each

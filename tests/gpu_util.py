@@ -36,4 +36,7 @@ def oracle_weights(block, branch_count):
                         norm2_w=block.norm2_weight[b].detach().float().cpu(),
                         wg=block.gate_weight[b].detach().float().cpu(), wu=block.up_weight[b].detach().float().cpu(),
                         wd=block.down_weight[b].detach().float().cpu()))
+        if getattr(block.attn, "qk_norm", False):
+            out[-1]["norm_q_w"] = block.attn.norm_q_weight[b].detach().float().cpu()
+            out[-1]["norm_k_w"] = block.attn.norm_k_weight[b].detach().float().cpu()
     return out

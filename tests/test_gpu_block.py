@@ -111,6 +111,39 @@ def test_mot_three_branch_block():
     assert_close(y3, y1.float().cpu(), 0.99999, 2e-3, "equal weights == single branch")
 
 
+def test_mot_block_with_qk_norm():
+    """Three-branch block with the per-head QK-RMSNorm switched on (own weight row per branch)."""
+    cfg = DMConfig("motn", 256, 2, 128, 512, 1, (2, 4, 8), n_text=40, n_action=24, n_branches=3, qk_norm=True)
+    st = DMStack(cfg, device=dev())
+    blk = st.blocks[0]
+    g = torch.Generator(device=dev()).manual_seed(21)
+    blk.reset_parameters(g)
+    with torch.no_grad():
+        blk.attn.norm_q_weight.copy_(1 + 0.3 * torch.randn(3, 128, generator=g, device=dev()))
+        blk.attn.norm_k_weight.copy_(1 + 0.3 * torch.randn(3, 128, generator=g, device=dev()))
+        blk.adaLN_modulation.bias.copy_(0.3 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
+    gc = torch.Generator().manual_seed(21)
+    x, xr = rand_bf16((cfg.n_tokens, 256), gc)
+    temb, tembr = rand_bf16((256,), gc)
+    segs = st.segments()
+    y = blk(x, temb, st.rotary(dev()), segs)
+    mod = O.adaln_modulation(tembr.view(1, -1), blk.adaLN_modulation.weight.float().cpu(),
+                             blk.adaLN_modulation.bias.float().cpu())
+    pos = O.joint_positions([("text", 40), ("video", cfg.grid), ("action", 24)])
+    cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+    ws = oracle_weights(blk, 3)
+    assert "norm_q_w" in ws[0]
+    want = O.dm_block(xr, ws, mod, cos, sin, 2, segs)
+    assert_close(y, want, BF16_COS, BF16_REL, "MoT block with QK-norm")
+    # a permuted segment order (video branch first in the table) must pick the same weight rows
+    y2 = blk(x, temb, st.rotary(dev()), [(0, 40, 0, False), (40, 64, 1, True), (104, 24, 2, True)])
+    assert torch.equal(y, y2)
+    # without the norm the result differs (the switch is live)
+    want_plain = O.dm_block(xr, [{k: v for k, v in w.items() if k not in ("norm_q_w", "norm_k_w")} for w in ws], mod, cos,
+                            sin, 2, segs)
+    assert O.max_rel_err(want, want_plain) > 1e-2
+
+
 def test_small_stack_and_encoder_path():
     cfg = DMConfig("s", 256, 4, 64, 640, 3, (2, 3, 10), n_text=20, mrope_sections=(16, 24, 24))
     st = DMStack(cfg, device=dev())

@@ -199,6 +199,40 @@ def test_attention_with_rope_in_registers(n, H, hd, sections, variant):
     assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"attention+rope n={n} hd={hd} variant={variant}")
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n,H,hd,seg_ends", [(300, 2, 128, (300,)), (130, 3, 64, (17, 100, 130)), (70, 1, 128, (64, 70))])
+def test_attention_with_qk_norm_and_rope(n, H, hd, seg_ends, variant):
+    """Per-head QK-RMSNorm (one weight row per token segment) ahead of the rotation, both inside the kernels."""
+    g = gen(n + 3 * hd)
+    d = H * hd
+    pos, _ = rotary.build_positions(n, (0, 0, 0), 0)
+    sections = (32, 48, 48) if hd == 128 else (16, 24, 24)
+    cos, sin = rotary.rotary_tables(pos, hd, sections)
+    qkv, qkvr = rand_bf16((n, 3 * d), g, 2.0)
+    ns = len(seg_ends)
+    qw = 1.0 + 0.3 * torch.randn(ns, hd, generator=g)
+    kw = 1.0 + 0.3 * torch.randn(ns, hd, generator=g)
+    prev = ops.set_variant("attn", variant)
+    try:
+        o = ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], H, hd, cos=cos.to(dev()), sin=sin.to(dev()),
+                          qk_norm=(qw.to(dev()), kw.to(dev()), seg_ends, 1e-6))
+    finally:
+        ops.set_variant("attn", prev)
+    qn, kn = torch.empty(n, H, hd), torch.empty(n, H, hd)
+    s0 = 0
+    for i, e in enumerate(seg_ends):
+        qn[s0:e] = O.rms_norm(qkvr[s0:e, :d].view(-1, H, hd), qw[i], 1e-6)
+        kn[s0:e] = O.rms_norm(qkvr[s0:e, d:2 * d].view(-1, H, hd), kw[i], 1e-6)
+        s0 = e
+    want = O.attention(O.apply_mrope(qn, cos, sin), O.apply_mrope(kn, cos, sin), qkvr[:, 2 * d:].view(n, H, hd))
+    assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"attention+qknorm+rope n={n} hd={hd} variant={variant}")
+    # scale invariance of RMSNorm: scaling Q and K changes nothing
+    o2 = ops.attention((qkv[:, :d].float() * 0.5).to(torch.bfloat16), (qkv[:, d:2 * d].float() * 4.0).to(torch.bfloat16),
+                       qkv[:, 2 * d:], H, hd, cos=cos.to(dev()), sin=sin.to(dev()),
+                       qk_norm=(qw.to(dev()), kw.to(dev()), seg_ends, 1e-6))
+    assert_close(o2, o.float().cpu(), 0.9999, 1e-2, "qk-norm scale invariance")
+
+
 def test_attention_closed_forms_and_determinism():
     g = gen(9)
     n, H, hd = 200, 2, 128
