@@ -1,5 +1,4 @@
-// Standalone rotate-half mRoPE on Q and K (in place) and the V transpose that feeds attention.
-// Both are HBM-bound streaming kernels.
+// Standalone rotate-half mRoPE on Q and K (in place): an HBM-bound streaming kernel.
 #include "cdm_common.h"
 
 namespace {

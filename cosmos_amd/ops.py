@@ -251,6 +251,35 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     return out
 
 
+def cfg_step(x: torch.Tensor, v_cond: torch.Tensor, v_uncond: Optional[torch.Tensor], guidance: float,
+             coef: Sequence[float], hist: Sequence[torch.Tensor] = (), v_out: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = coef[0] x + coef[1] v + sum_i coef[2+i] hist[i], v = v_uncond + guidance (v_cond - v_uncond)
+    (v = v_cond without v_uncond).  x, out, hist, v_out: fp32; v_cond, v_uncond: bf16; all of one shape, contiguous.
+    ``out`` may be ``x`` itself."""
+    lib = _lib.load()
+    n = x.numel()
+    if len(coef) != 2 + len(hist):
+        raise ValueError("coef must hold 2 + len(hist) values")
+    for t, name, dt in [(x, "x", torch.float32), (v_cond, "v_cond", torch.bfloat16)] + \
+                       ([(v_uncond, "v_uncond", torch.bfloat16)] if v_uncond is not None else []) + \
+                       [(h, "hist", torch.float32) for h in hist] + \
+                       ([(v_out, "v_out", torch.float32)] if v_out is not None else []):
+        if t.numel() != n or not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous with {n} elements")
+        _chk(t.reshape(-1), name, dt)
+    if out is None:
+        out = torch.empty_like(x)
+    _chk(out.reshape(-1), "out", torch.float32)
+    hp = (C.c_void_p * max(len(hist), 1))(*[h.data_ptr() for h in hist])
+    cf = (C.c_float * len(coef))(*[float(c) for c in coef])
+    rc = lib.cdm_cfg_step_f32(x.data_ptr(), v_cond.data_ptr(), v_uncond.data_ptr() if v_uncond is not None else None,
+                              float(guidance), hp, cf, len(hist), v_out.data_ptr() if v_out is not None else None,
+                              out.data_ptr(), n, _stream())
+    _lib.check(rc, "cdm_cfg_step_f32")
+    return out
+
+
 _ATTN_TIMER = None
 
 

@@ -198,6 +198,22 @@ int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, 
  * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default. */
 int32_t cdm_set_variant(const char* op, int32_t variant);
 
+/*
+ * Classifier-free-guidance combine fused with the scheduler's linear latent update - replaces, inside one
+ * denoising iteration of the pipeline (Cosmos3OmniPipeline.__call__, README.md:249-263: guidance_scale;
+ * README.md:247: UniPCMultistepScheduler with flow_shift), the elementwise tail
+ *     v   = v_uncond + guidance * (v_cond - v_uncond)            (v = v_cond when v_uncond is null)
+ *     out = coef[0] * x + coef[1] * v + sum_i coef[2 + i] * hist[i]
+ * which is the form of an Euler flow-matching step (coef = {1, sigma_next - sigma}) and of every linear multistep
+ * update (UniPC, DPM-Solver++): the scheduler computes the scalar coefficients on the host, this kernel makes one
+ * pass over the tensors.  x, out, hist[i], v_out: fp32 [n]; v_cond, v_uncond: bf16 [n] (the transformer's output);
+ * v_out (optional) receives v, the model output a multistep scheduler keeps as history; out may alias x.
+ * hist and coef are HOST arrays (n_hist <= 4 device pointers; 2 + n_hist floats).
+ */
+int32_t cdm_cfg_step_f32(const float* x, const void* v_cond, const void* v_uncond, float guidance,
+                         const float* const* hist, const float* coef, int32_t n_hist, float* v_out, float* out,
+                         int64_t n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,12 +23,15 @@ closed forms / float64 brute force (tests/test_oracle_*.py):
 pinned by closed forms and float64 brute force only (no library routine
 exists for them):
     adaln_rms_norm modulation, gated residual, MoT segment routing,
-    e4m3 quantisation (against torch.float8_e4m3fn casts).
+    e4m3 quantisation (against torch.float8_e4m3fn casts), cfg_step (guidance
+    combine + linear scheduler update).
 parity unpinned against the real Cosmos 3 generator (only an import of the
 absent diffusers implementation could pin them; the benchmark configuration
 text governs instead):
     timestep_embedding / time_mlp conventions, adaLN chunk order and the
     (1 + scale) convention, mRoPE channel layout choice (chunked is the
-    default), modality position offsets in generator mode, the fp8 recipe.
+    default), modality position offsets in generator mode, the fp8 recipe,
+    the scheduler's coefficient rule (flow_sigmas is the plain shifted Euler
+    schedule; the reference's UniPC coefficients live in diffusers).
 """
 from .dm_oracle import *  # noqa: F401,F403

@@ -21,7 +21,7 @@ __all__ = [
     "mrope_axis_map", "text_positions", "vision_positions", "joint_positions",
     "mrope_cos_sin", "apply_mrope", "attention", "attention_rows", "swiglu",
     "dm_block", "dm_stack", "quant_e4m3_rows", "quant_e4m3_weight", "fp8_linear",
-    "max_rel_err", "cos_sim", "E4M3_MAX",
+    "max_rel_err", "cos_sim", "E4M3_MAX", "cfg_step", "flow_sigmas",
 ]
 
 E4M3_MAX = 448.0
@@ -333,6 +333,29 @@ def dm_stack(x, blocks: Sequence[Sequence[Dict[str, torch.Tensor]]], mods: Seque
 # --------------------------------------------------------------------------
 # error measures used by every parity test
 # --------------------------------------------------------------------------
+def cfg_step(x, v_cond, v_uncond, guidance: float, coef: Sequence[float], hist: Sequence[torch.Tensor] = ()):
+    """Guidance combine + linear scheduler update, fp32:
+        v = v_uncond + guidance (v_cond - v_uncond)        (v = v_cond without v_uncond)
+        out = coef[0] x + coef[1] v + sum_i coef[2+i] hist[i]
+    Returns (out, v).  The reference sets guidance_scale and a flow-shifted multistep scheduler at its call site
+    (README.md:247,258); the combine is the standard classifier-free-guidance formula, and every linear multistep
+    scheduler update has this form once its scalar coefficients are known.  Pinned by closed forms only
+    (guidance 1 -> v_cond, guidance 0 -> v_uncond, linearity)."""
+    vc = v_cond.to(torch.float32)
+    v = vc if v_uncond is None else v_uncond.to(torch.float32) + guidance * (vc - v_uncond.to(torch.float32))
+    out = coef[0] * x.to(torch.float32) + coef[1] * v
+    for c, h in zip(coef[2:], hist):
+        out = out + c * h.to(torch.float32)
+    return out, v
+
+
+def flow_sigmas(num_steps: int, flow_shift: float = 1.0) -> torch.Tensor:
+    """Flow-matching noise levels 1 -> 0 in ``num_steps`` steps with the time shift
+    sigma' = shift sigma / (1 + (shift - 1) sigma)  (the ``flow_shift`` of README.md:247); float64."""
+    s = torch.linspace(1.0, 0.0, num_steps + 1, dtype=torch.float64)
+    return flow_shift * s / (1.0 + (flow_shift - 1.0) * s)
+
+
 def max_rel_err(a: torch.Tensor, b: torch.Tensor) -> float:
     """max|a-b| / max|b| over the whole tensor (b = oracle)."""
     a = a.detach().to(torch.float64).cpu(); b = b.detach().to(torch.float64).cpu()

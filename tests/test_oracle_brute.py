@@ -162,3 +162,24 @@ def test_e4m3_quant():
     c2 = (q * s) @ (wq * sw).t()
     assert torch.allclose(c1, c2, rtol=1e-4, atol=1e-3)
     assert O.max_rel_err(c1[:4], a[:4] @ w.t()) < 5e-2
+
+
+def test_cfg_step_closed_forms():
+    g = torch.Generator().manual_seed(1)
+    x, vc, vu, h = (torch.randn(64, generator=g) for _ in range(4))
+    out, v = O.cfg_step(x, vc, vu, 1.0, [0.0, 1.0])
+    assert torch.allclose(out, vc, atol=1e-6) and torch.allclose(v, vc, atol=1e-6)           # guidance 1 -> cond
+    assert torch.equal(O.cfg_step(x, vc, vu, 0.0, [0.0, 1.0])[0], vu)                        # guidance 0 -> uncond
+    assert torch.equal(O.cfg_step(x, vc, None, 9.0, [1.0, 0.0])[0], x)                       # no update
+    # the guided prediction extrapolates: v - vu = g (vc - vu)
+    _, v6 = O.cfg_step(x, vc, vu, 6.0, [1.0, 0.0])
+    assert torch.allclose(v6 - vu, 6.0 * (vc - vu), atol=1e-5)
+    # linear in every tensor and coefficient (float64 brute force)
+    want = (0.5 * x.double() - 0.25 * (vu.double() + 2.0 * (vc.double() - vu.double())) + 0.125 * h.double())
+    got, _ = O.cfg_step(x, vc, vu, 2.0, [0.5, -0.25, 0.125], [h])
+    assert torch.allclose(got.double(), want, atol=1e-6)
+    # noise levels: endpoints, monotone, shift 1 = uniform grid, shift identity sigma' (1 + (s-1) sigma) = s sigma
+    s1, s3 = O.flow_sigmas(10, 1.0), O.flow_sigmas(10, 3.0)
+    assert s1[0] == 1.0 and s1[-1] == 0.0 and torch.allclose(s1, torch.linspace(1, 0, 11, dtype=torch.float64))
+    assert s3[0] == 1.0 and s3[-1] == 0.0 and bool((s3[1:] < s3[:-1]).all()) and bool((s3[1:-1] > s1[1:-1]).all())
+    assert torch.allclose(s3 * (1 + 2.0 * s1), 3.0 * s1)
