@@ -402,3 +402,108 @@ class DMStack(nn.Module):
         if return_dict:
             return {"sample": out, "joint": x}
         return (out,)
+
+
+class DMTransformer(nn.Module):
+    """The transformer-shaped object a diffusers pipeline drives (``pipe.transformer``): latents in, velocity out.
+
+    Stack edges around ``DMStack``: patchify + ``proj_in``, the block stack, a final RMSNorm, ``proj_out`` +
+    unpatchify; an optional action stream (``action_proj_in`` + ``action_modality_embed`` in, ``action_proj_out``
+    out).  The edge linears are one-off projections with K or N = patch width (64 for 16 latent channels and 1x2x2
+    patches): 0.1 % of a step's flops, they stay on the stock BLAS path like the one-row timestep MLP.  Parameter
+    names follow the checkpoint keys the reference's model files attest (``proj_in``, ``proj_out``,
+    ``time_embedder``, ``action_proj_in``, ``action_proj_out``, ``action_modality_embed``); the patch order
+    (channel-major inside a patch) and the un-modulated final norm are this build's choices.
+    """
+
+    def __init__(self, cfg: DMConfig, latent_channels: int = 16, patch: Tuple[int, int, int] = (1, 2, 2),
+                 action_dim: int = 0, device=None, dtype=torch.bfloat16):
+        super().__init__()
+        self.cfg, self.latent_channels, self.patch, self.action_dim = cfg, latent_channels, tuple(patch), action_dim
+        pd = latent_channels * patch[0] * patch[1] * patch[2]
+        self.stack = DMStack(cfg, device=device, dtype=dtype)
+        self.proj_in = nn.Linear(pd, cfg.d_model, device=device, dtype=dtype)
+        self.proj_out = nn.Linear(cfg.d_model, pd, device=device, dtype=dtype)
+        self.norm_out = nn.Parameter(torch.ones(cfg.d_model, device=device, dtype=dtype), requires_grad=False)
+        if cfg.n_action:
+            if action_dim <= 0:
+                raise ValueError("a configuration with action tokens needs action_dim")
+            self.action_proj_in = nn.Linear(action_dim, cfg.d_model, device=device, dtype=dtype)
+            self.action_proj_out = nn.Linear(cfg.d_model, action_dim, device=device, dtype=dtype)
+            self.action_modality_embed = nn.Parameter(torch.zeros(cfg.d_model, device=device, dtype=dtype),
+                                                      requires_grad=False)
+        for p in self.parameters():
+            p.requires_grad_(False)
+
+    @property
+    def time_embedder(self):
+        return self.stack.time_embedder
+
+    @torch.no_grad()
+    def reset_parameters(self, seed: Optional[int] = None) -> None:
+        self.stack.reset_parameters(seed)
+        dev = self.proj_in.weight.device
+        g = torch.Generator(device=dev).manual_seed((self.cfg.seed if seed is None else seed) + 7919)
+        mods = [self.proj_in, self.proj_out] + ([self.action_proj_in, self.action_proj_out] if self.cfg.n_action else [])
+        for m in mods:
+            m.weight.copy_((torch.randn(m.weight.shape, generator=g, device=dev) * 0.02).to(m.weight.dtype))
+            m.bias.zero_()
+
+    # ---- patch layout: token (t, h, w) of the grid holds the latent patch [C, pt, ph, pw] flattened channel-major
+    def patchify(self, latents: torch.Tensor) -> torch.Tensor:
+        C, (pt, ph, pw) = self.latent_channels, self.patch
+        T, H, W = self.cfg.grid
+        x = latents.reshape(C, T, pt, H, ph, W, pw).permute(1, 3, 5, 0, 2, 4, 6)
+        return x.reshape(T * H * W, C * pt * ph * pw)
+
+    def unpatchify(self, tokens: torch.Tensor) -> torch.Tensor:
+        C, (pt, ph, pw) = self.latent_channels, self.patch
+        T, H, W = self.cfg.grid
+        x = tokens.reshape(T, H, W, C, pt, ph, pw).permute(3, 0, 4, 1, 5, 2, 6)
+        return x.reshape(1, C, T * pt, H * ph, W * pw)
+
+    @torch.no_grad()
+    def forward(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
+                encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
+                return_dict: bool = False):
+        """hidden_states: latents [1, C, T*pt, H*ph, W*pw]; encoder_hidden_states: [1, n_text, d] context already in
+        model width; action_states: [1, n_action, action_dim].  Returns the velocity prediction, latents-shaped and
+        bf16 (plus the action prediction when there is an action stream)."""
+        c = self.cfg
+        dt = self.proj_in.weight.dtype
+        tok = self.proj_in(self.patchify(hidden_states[0].to(dt)))
+        act = None
+        if c.n_action:
+            if action_states is None:
+                raise ValueError("this configuration expects action_states")
+            act = self.action_proj_in(_as2d(action_states).to(dt)) + self.action_modality_embed
+        res = self.stack(tok, timestep, encoder_hidden_states=encoder_hidden_states, action_states=act, return_dict=True)
+        joint = res["joint"]
+        y = ops.adaln_rmsnorm(joint, self.norm_out.data, None, None, c.eps)
+        video = y[c.n_text:c.n_text + c.n_video]
+        sample = self.unpatchify(self.proj_out(video))
+        out_act = self.action_proj_out(y[c.n_text + c.n_video:]).unsqueeze(0) if c.n_action else None
+        if return_dict:
+            return {"sample": sample, "action": out_act}
+        return (sample,) if out_act is None else (sample, out_act)
+
+    # ---- checkpoint plumbing (see cosmos_amd.checkpoint)
+    def _top(self):
+        mods = {"proj_in": self.proj_in, "proj_out": self.proj_out, "time_embedder.linear_1": self.stack.time_embedder.linear_1,
+                "time_embedder.linear_2": self.stack.time_embedder.linear_2}
+        if self.cfg.n_action:
+            mods.update({"action_proj_in": self.action_proj_in, "action_proj_out": self.action_proj_out})
+        t = {f"{k}.{p}": getattr(m, p) for k, m in mods.items() for p in ("weight", "bias")}
+        t["norm_out.weight"] = self.norm_out
+        if self.cfg.n_action:
+            t["action_modality_embed"] = self.action_modality_embed
+        return t
+
+    def top_level_keys(self) -> List[str]:
+        return list(self._top())
+
+    def assign_top_level(self, key: str, t: torch.Tensor) -> None:
+        self._top()[key].data.copy_(t)
+
+    def export_top_level(self):
+        return {k: p.data.clone() for k, p in self._top().items()}

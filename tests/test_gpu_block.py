@@ -235,3 +235,60 @@ def test_c1_full_size_attention_sampled_rows():
     vmin, vmax = v.float().amin(0), v.float().amax(0)
     of = o.float()
     assert bool((of >= vmin - 1e-2).all()) and bool((of <= vmax + 1e-2).all())
+
+
+def test_transformer_with_stack_edges_and_loaded_checkpoint(tmp_path):
+    """latents -> patchify/proj_in -> 2 MoT blocks (QK-norm) -> final norm -> proj_out/unpatchify, with the weights
+    taken through a safetensors file; checked against the fp32 oracle composed from the same tensors."""
+    from safetensors.torch import save_file
+    from cosmos_amd import DMTransformer, export_generator_weights, load_generator_weights
+    cfg = DMConfig("edge", 256, 2, 128, 512, 2, (2, 3, 4), n_text=12, n_action=5, n_branches=3, qk_norm=True)
+    src = DMTransformer(cfg, latent_channels=4, action_dim=6, device=dev())
+    src.reset_parameters(31)
+    g = torch.Generator(device=dev()).manual_seed(31)
+    with torch.no_grad():
+        for blk in src.stack.blocks:
+            blk.attn.norm_q_weight.copy_(1 + 0.2 * torch.randn(3, 128, generator=g, device=dev()))
+            blk.attn.norm_k_weight.copy_(1 + 0.2 * torch.randn(3, 128, generator=g, device=dev()))
+            blk.adaLN_modulation.bias.copy_(0.2 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
+        src.norm_out.copy_(1 + 0.2 * torch.randn(256, generator=g, device=dev()))
+        src.action_modality_embed.copy_(0.5 * torch.randn(256, generator=g, device=dev()))
+    # the third (action) branch has no attested key names: it travels as the DM names of an extra mapping
+    path = str(tmp_path / "gen.safetensors")
+    save_file({k: v.contiguous().cpu() for k, v in export_generator_weights(src).items()}, path)
+    m = DMTransformer(cfg, latent_channels=4, action_dim=6, device=dev())
+    m.reset_parameters(99)
+    rep = load_generator_weights(m, path)
+    assert not rep["unexpected"] and all(".2" in k for k in rep["missing"])     # only branch 2 is absent from the file
+    with torch.no_grad():
+        for bs, bm in zip(src.stack.blocks, m.stack.blocks):
+            for name in ("norm1_weight", "norm2_weight", "gate_weight", "up_weight", "down_weight"):
+                getattr(bm, name)[2].copy_(getattr(bs, name)[2])
+            bm.attn.qkv_weight[2].copy_(bs.attn.qkv_weight[2]); bm.attn.out_weight[2].copy_(bs.attn.out_weight[2])
+            bm.attn.norm_q_weight[2].copy_(bs.attn.norm_q_weight[2]); bm.attn.norm_k_weight[2].copy_(bs.attn.norm_k_weight[2])
+    gc = torch.Generator().manual_seed(32)
+    lat = torch.randn(1, 4, 2, 6, 8, generator=gc)
+    ctx, ctxr = rand_bf16((1, 12, 256), gc)
+    act, actr = rand_bf16((1, 5, 6), gc)
+    t = torch.tensor([640.0])
+    out = m(lat.to(dev()), t.to(dev()), encoder_hidden_states=ctx, action_states=act, return_dict=True)
+    out_src = src(lat.to(dev()), t.to(dev()), encoder_hidden_states=ctx, action_states=act, return_dict=True)
+    assert torch.equal(out["sample"], out_src["sample"])            # the file carried every tensor exactly
+    # oracle composition (fp32)
+    f = lambda p: p.detach().float().cpu()
+    latb = lat.to(torch.bfloat16).float()
+    tok = m.patchify(latb[0]) @ f(m.proj_in.weight).t() + f(m.proj_in.bias)
+    a_in = actr[0] @ f(m.action_proj_in.weight).t() + f(m.action_proj_in.bias) + f(m.action_modality_embed)
+    x = torch.cat([ctxr[0], tok, a_in])
+    te = m.time_embedder
+    c = O.time_mlp(O.timestep_embedding(t), f(te.linear_1.weight), f(te.linear_1.bias), f(te.linear_2.weight), f(te.linear_2.bias))
+    mods = [O.adaln_modulation(c, f(b.adaLN_modulation.weight), f(b.adaLN_modulation.bias)) for b in m.stack.blocks]
+    pos = O.joint_positions([("text", 12), ("video", cfg.grid), ("action", 5)])
+    cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+    y = O.dm_stack(x, [oracle_weights(b, 3) for b in m.stack.blocks], mods, cos, sin, 2, m.stack.segments())
+    y = O.rms_norm(y, f(m.norm_out), cfg.eps)
+    want = m.unpatchify(y[12:12 + cfg.n_video] @ f(m.proj_out.weight).t() + f(m.proj_out.bias))
+    assert out["sample"].shape == lat.shape
+    assert_close(out["sample"], want, BF16_COS, BF16_REL, "transformer with stack edges")
+    want_act = y[12 + cfg.n_video:] @ f(m.action_proj_out.weight).t() + f(m.action_proj_out.bias)
+    assert_close(out["action"][0], want_act, BF16_COS, BF16_REL, "action head")
