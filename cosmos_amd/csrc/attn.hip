@@ -112,7 +112,7 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
                                           f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
-                                          bool next_ragged, int next_keys_valid) {
+                                          bool next_masked, const int (&next_keys_valid)[QS]) {
     constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
     // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot and
     // their result is never used - cheaper than a second copy of the step.)
@@ -167,9 +167,9 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
     for (int qs = 0; qs < QS; ++qs)
         asm volatile("" : "+v"(pf[qs][0]), "+v"(pf[qs][1]), "+v"(pf[qs][2]), "+v"(pf[qs][3]), "+v"(l_run[qs]));
     __builtin_amdgcn_sched_barrier(0);
-    if (next_ragged) {     // wave-uniform; only before a ragged last tile
+    if (next_masked) {     // wave-uniform: before a ragged last tile, and in every step of a causal query block
 #pragma unroll
-        for (int qs = 0; qs < QS; ++qs) mask_scores(s_next[qs], next_keys_valid, lane);
+        for (int qs = 0; qs < QS; ++qs) mask_scores(s_next[qs], next_keys_valid[qs], lane);
     }
 
     // ---- block B
@@ -234,6 +234,10 @@ struct PackedParams {
     const bf16_t* q; int64_t ldq;
     const char* kp;              // [n_heads][n_tiles][tile bytes]
     const char* vp;
+    const char* kp_prefix;       // optional tile images of keys that precede those of kp / vp (whole tiles)
+    const char* vp_prefix;
+    int n_prefix_tiles;
+    int causal_prefix;           // query rows < causal_prefix see keys <= their own index only; the others see all keys
     bf16_t* o; int64_t ldo;
     const float* cos; const float* sin;   // optional rotary tables [n_tokens, HD/2] applied to Q at load
     QkNormDev qn;                          // optional per-head RMSNorm of Q, applied before the rotation
@@ -340,28 +344,46 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             for (int v = 0; v < 16; ++v) oacc[qs][t][v] = 0.0f;
     }
 
-    const int NT = (p.n_tokens + BN - 1) / BN;
-    const int last_valid = p.n_tokens - (NT - 1) * BN;
+    // key tiles: NP whole tiles of the prefix images, then the NM tiles of the main images
+    const int NP = p.n_prefix_tiles, NM = (p.n_tokens + BN - 1) / BN;
+    const int NT = NP + NM;
+    const int n_keys = NP * BN + p.n_tokens;
+    const int last_valid = n_keys - (NT - 1) * BN;
+    // per-row key limit and the tiles this workgroup needs: a query block inside the causal prefix stops at its
+    // own last row, and every tile it visits is masked per row
+    const int b0 = blockIdx.x * BMQ;
+    const bool causal_wg = b0 < p.causal_prefix;
+    int klim[QS];
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs) {
+        const int qrow = q0 + qs * 32 + r32;
+        klim[qs] = qrow < p.causal_prefix ? qrow + 1 : n_keys;
+    }
+    const int kmax = (causal_wg && b0 + BMQ <= p.causal_prefix) ? (b0 + BMQ < n_keys ? b0 + BMQ : n_keys) : n_keys;
+    const int NTW = (kmax + BN - 1) / BN;
     const uint32_t lane_off = (uint32_t)(wave * 1024 + lane * 16);
-    const char* kbase = p.kp + (int64_t)head * NT * TILE_BYTES;
-    const char* vbase = p.vp + (int64_t)head * NT * TILE_BYTES;
+    const char* kbase = p.kp + (int64_t)head * NM * TILE_BYTES;
+    const char* vbase = p.vp + (int64_t)head * NM * TILE_BYTES;
+    const char* kpre = p.kp_prefix + (int64_t)head * NP * TILE_BYTES;
+    const char* vpre = p.vp_prefix + (int64_t)head * NP * TILE_BYTES;
     const uint32_t sk_addr = lds_addr_of(sk) + wave * 1024, sv_addr = lds_addr_of(sv) + wave * 1024;
 
     // tile `t` (clamped to the last tile, so that every step issues the same number of loads and the
     // vmcnt arithmetic below stays valid at the end of the sequence) -> ring slot `slot`
-    auto issue = [&](const char* base, uint32_t dst_addr, int t, int slot) {
-        const char* src = base + (int64_t)(t < NT ? t : NT - 1) * TILE_BYTES;
+    auto issue = [&](const char* base, const char* pre, uint32_t dst_addr, int t, int slot) {
+        const int tc = t < NT ? t : NT - 1;
+        const char* src = tc < NP ? pre + (int64_t)tc * TILE_BYTES : base + (int64_t)(tc - NP) * TILE_BYTES;
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i)
             lds_dma16(src + i * (NW * 1024), lane_off, dst_addr + slot * TILE_BYTES + i * (NW * 1024));
     };
 
     // ---- prologue: K(0) | K(1), V(0) | K(2), V(1); scores of tile 0 with an exact first reference
-    issue(kbase, sk_addr, 0, 0);
-    issue(kbase, sk_addr, 1, 1);
-    issue(vbase, sv_addr, 0, 0);
-    issue(kbase, sk_addr, 2, 2);
-    issue(vbase, sv_addr, 1, 1);
+    issue(kbase, kpre, sk_addr, 0, 0);
+    issue(kbase, kpre, sk_addr, 1, 1);
+    issue(vbase, vpre, sv_addr, 0, 0);
+    issue(kbase, kpre, sk_addr, 2, 2);
+    issue(vbase, vpre, sv_addr, 1, 1);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
     f32x16 s_a[QS][2], s_b[QS][2];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
@@ -370,7 +392,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s_a[qs][0][v] = 0.0f; s_a[qs][1][v] = 0.0f; }
         scores_tile<HD>(sk, qf[qs], s_a[qs], lane);
-        if (NT == 1 && ragged) mask_scores(s_a[qs], last_valid, lane);
+        if (causal_wg || (NT == 1 && ragged)) mask_scores(s_a[qs], klim[qs], lane);
         const float m0 = tile_row_max(s_a[qs]);      // exact first reference: every row has at least one finite score
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -392,17 +414,19 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory");                           \
         const int k_fill = vs_cur;                              /* slot of K(j)   == j % 3     */               \
         const int v_fill = ks_next == 2 ? 0 : ks_next + 1;      /* slot of V(j-1) == (j+2) % 3 */               \
-        issue(kbase, sk_addr, j + 3, k_fill);                                                                   \
-        issue(vbase, sv_addr, j + 2, v_fill);                                                                   \
+        issue(kbase, kpre, sk_addr, j + 3, k_fill);                                                             \
+        issue(vbase, vpre, sv_addr, j + 2, v_fill);                                                             \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
+        int nvalid[QS];                                                                                         \
+        _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
         pipe_step<HD, QS>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,  \
-                          SCUR, SNEXT, oacc, negm, l_run, lane, ragged && j + 2 == NT, last_valid);            \
+                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 == NT), nvalid);  \
         vs_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
-    for (int j = 0; j < NT; ++j) {
+    for (int j = 0; j < NTW; ++j) {
         CDM_ATTN_STEP(s_a, s_b)
-        if (++j >= NT) break;
+        if (++j >= NTW) break;
         CDM_ATTN_STEP(s_b, s_a)
     }
 #undef CDM_ATTN_STEP
@@ -592,8 +616,17 @@ extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void*
 extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
                                             const void* workspace, void* o, int64_t ldo, int64_t n_tokens,
                                             int32_t n_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
-                                            void* stream) {
+                                            const void* prefix_workspace, int64_t n_prefix_tokens,
+                                            int64_t causal_prefix, void* stream) {
     CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
+    CDM_REQUIRE(n_prefix_tokens >= 0 && n_prefix_tokens % BN == 0 && n_prefix_tokens < (1ll << 23), CDM_ERR_BAD_SHAPE,
+                "attn_fwd_packed: n_prefix_tokens=%lld must be a non-negative multiple of %d", (long long)n_prefix_tokens, BN);
+    CDM_REQUIRE((n_prefix_tokens > 0) == (prefix_workspace != nullptr) && cdm_aligned16(prefix_workspace), CDM_ERR_BAD_ARG,
+                "attn_fwd_packed: prefix_workspace and n_prefix_tokens must be given together (16-byte aligned)");
+    CDM_REQUIRE(causal_prefix >= 0 && causal_prefix <= n_tokens, CDM_ERR_BAD_ARG,
+                "attn_fwd_packed: causal_prefix=%lld outside [0, n_tokens]", (long long)causal_prefix);
+    CDM_REQUIRE(causal_prefix == 0 || n_prefix_tokens == 0, CDM_ERR_UNSUPPORTED,
+                "attn_fwd_packed: a causal prefix cannot be combined with prefix key images");
     int32_t rc = check_attn_common("attn_fwd_packed", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
     QkNormDev qn;
@@ -608,6 +641,10 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     PackedParams p;
     p.q = (const bf16_t*)q; p.ldq = ldq;
     p.kp = (const char*)workspace; p.vp = (const char*)workspace + img;
+    p.kp_prefix = (const char*)prefix_workspace;
+    p.vp_prefix = (const char*)prefix_workspace + image_bytes(n_prefix_tokens, n_heads, head_dim);
+    p.n_prefix_tiles = (int)(n_prefix_tokens / BN);
+    p.causal_prefix = (int)causal_prefix;
     p.o = (bf16_t*)o; p.ldo = ldo;
     p.cos = cos; p.sin = sin;
     p.qn = qn;
@@ -629,7 +666,8 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
 extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                                      int64_t ldv, const float* cos, const float* sin, void* o, int64_t ldo,
                                      int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* workspace,
-                                     int64_t workspace_bytes, const cdm_qk_norm* qk_norm, void* stream) {
+                                     int64_t workspace_bytes, const cdm_qk_norm* qk_norm, int64_t causal_prefix,
+                                     void* stream) {
     CDM_REQUIRE(q && k && v && o, CDM_ERR_BAD_ARG, "attn_fwd: null pointer");
     int32_t rc = check_attn_common("attn_fwd", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
@@ -644,11 +682,14 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
     // validate the second stage's arguments before the first stage is enqueued
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldq >= d && ldk >= d && ldv >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd: row stride smaller than n_heads*head_dim");
+    CDM_REQUIRE(causal_prefix >= 0 && causal_prefix <= n_tokens, CDM_ERR_BAD_ARG,
+                "attn_fwd: causal_prefix=%lld outside [0, n_tokens]", (long long)causal_prefix);
     CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(o) && ldq % 8 == 0 &&
                     ldk % 8 == 0 && ldv % 8 == 0 && ldo % 4 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
     if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_heads, head_dim,
                                     qk_norm, stream)))
         return rc;
-    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, head_dim, qk_norm, stream);
+    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, head_dim, qk_norm, nullptr,
+                                    0, causal_prefix, stream);
 }

@@ -203,14 +203,81 @@ def attn_workspace_bytes(n_tokens: int, n_heads: int, head_dim: int) -> int:
     return int(_lib.load().cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim))
 
 
+def _qk_norm_arg(qk_norm, head_dim: int):
+    """-> (pointer or None, keep-alive objects) for the optional ``cdm_qk_norm`` argument."""
+    if qk_norm is None:
+        return None, None
+    qw, kw, seg_ends, eps = qk_norm
+    seg_ends = [int(e) for e in seg_ends]
+    ends = (C.c_int64 * len(seg_ends))(*seg_ends)
+    st = _lib.QkNorm(_f32vec(qw, "qk_norm q_weight", len(seg_ends) * head_dim),
+                     _f32vec(kw, "qk_norm k_weight", len(seg_ends) * head_dim), ends, len(seg_ends), float(eps))
+    return C.addressof(st), (st, ends)
+
+
+def attention_pack_kv(k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
+                      workspace: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
+                      sin: Optional[torch.Tensor] = None, qk_norm=None) -> torch.Tensor:
+    """First stage of ``attention``: K (normalised / rotated if asked) and V of ``n`` tokens -> tile images in
+    ``workspace`` (returned).  The images can be kept and passed to ``attention_packed`` as its ``prefix``."""
+    lib = _lib.load()
+    n, d = k.shape[0], n_heads * head_dim
+    if k.shape != (n, d) or v.shape != (n, d):
+        raise ValueError("k, v must be [n_tokens, n_heads*head_dim]")
+    if workspace is None:
+        workspace = torch.empty((max(attn_workspace_bytes(n, n_heads, head_dim), 16),), dtype=torch.uint8, device=k.device)
+    half = head_dim // 2
+    qn, _keep = _qk_norm_arg(qk_norm, head_dim)
+    rc = lib.cdm_attn_pack_kv_bf16(_chk(k, "k", torch.bfloat16, 2), k.stride(0), _chk(v, "v", torch.bfloat16, 2),
+                                   v.stride(0), _f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half),
+                                   _chk(workspace, "workspace", torch.uint8, 1), workspace.numel(), n, n_heads, head_dim,
+                                   qn, _stream())
+    _lib.check(rc, "cdm_attn_pack_kv_bf16")
+    return workspace
+
+
+def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, head_dim: int,
+                     out: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
+                     sin: Optional[torch.Tensor] = None, qk_norm=None, prefix=None,
+                     causal_prefix: int = 0) -> torch.Tensor:
+    """Second stage of ``attention``: the ``n`` query rows against the keys packed in ``workspace`` (``n`` tokens),
+    preceded by the keys of ``prefix`` = (images, n_prefix_tokens) if given."""
+    lib = _lib.load()
+    n, d = q.shape[0], n_heads * head_dim
+    if out is None:
+        out = torch.empty((n, d), dtype=torch.bfloat16, device=q.device)
+    half = head_dim // 2
+    qn, _keep = _qk_norm_arg(qk_norm, head_dim)
+    pws, npre = (None, 0) if prefix is None else (_chk(prefix[0], "prefix images", torch.uint8, 1), int(prefix[1]))
+    if prefix is not None and prefix[0].numel() < attn_workspace_bytes(npre, n_heads, head_dim):
+        raise ValueError("prefix images are smaller than the workspace of n_prefix tokens")
+    if workspace.numel() < attn_workspace_bytes(n, n_heads, head_dim):
+        raise ValueError("workspace is smaller than the images of n tokens")
+    timer = _ATTN_TIMER
+    if timer is not None:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+    rc = lib.cdm_attn_fwd_packed_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _f32vec(cos, "cos", n * half),
+                                      _f32vec(sin, "sin", n * half), _chk(workspace, "workspace", torch.uint8, 1),
+                                      _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, head_dim, qn, pws,
+                                      npre, int(causal_prefix), _stream())
+    if timer is not None:
+        e1.record()
+        timer.append((e0, e1))
+    _lib.check(rc, "cdm_attn_fwd_packed_bf16")
+    return out
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
               out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
               cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
-              qk_norm=None) -> torch.Tensor:
-    """Full non-causal attention; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free).
+              qk_norm=None, causal_prefix: int = 0, prefix=None) -> torch.Tensor:
+    """Attention over the joint sequence; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free).
     With cos/sin ([n, head_dim/2] fp32) rotate-half mRoPE is applied to Q and K inside the kernels.
     ``qk_norm`` = (q_weight, k_weight, seg_ends, eps) switches on the per-head RMSNorm of Q and K ahead of the
-    rotation: weights [n_seg, head_dim] fp32 on the device, ``seg_ends`` the exclusive end token of each segment."""
+    rotation: weights [n_seg, head_dim] fp32 on the device, ``seg_ends`` the exclusive end token of each segment.
+    ``causal_prefix`` = P > 0 selects the hybrid mask (the first P tokens causal among themselves, blind to the
+    rest; all others see everything); ``prefix`` = (images, n_prefix_tokens) prepends already packed keys."""
     lib = _lib.load()
     n = q.shape[0]
     d = n_heads * head_dim
@@ -221,34 +288,20 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     need = attn_workspace_bytes(n, n_heads, head_dim)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
-    half = head_dim // 2
-    qp, kp, vp = _chk(q, "q", torch.bfloat16, 2), _chk(k, "k", torch.bfloat16, 2), _chk(v, "v", torch.bfloat16, 2)
-    op, wp = _chk(out, "out", torch.bfloat16, 2), _chk(workspace, "workspace", torch.uint8, 1)
-    cp, sp = _f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half)
-    qn = None
-    if qk_norm is not None:
-        qw, kw, seg_ends, eps = qk_norm
-        seg_ends = [int(e) for e in seg_ends]
-        ends = (C.c_int64 * len(seg_ends))(*seg_ends)
-        qn_struct = _lib.QkNorm(_f32vec(qw, "qk_norm q_weight", len(seg_ends) * head_dim),
-                                _f32vec(kw, "qk_norm k_weight", len(seg_ends) * head_dim), ends, len(seg_ends), float(eps))
-        qn = C.addressof(qn_struct)        # qn_struct and ends stay alive until the calls below have returned
-    if _ATTN_TIMER is None:
-        rc = lib.cdm_attn_fwd_bf16(qp, q.stride(0), kp, k.stride(0), vp, v.stride(0), cp, sp, op, out.stride(0), n,
-                                   n_heads, head_dim, wp, workspace.numel(), qn, _stream())
+    if _ATTN_TIMER is None and prefix is None:
+        half = head_dim // 2
+        qn, _keep = _qk_norm_arg(qk_norm, head_dim)
+        rc = lib.cdm_attn_fwd_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _chk(k, "k", torch.bfloat16, 2),
+                                   k.stride(0), _chk(v, "v", torch.bfloat16, 2), v.stride(0),
+                                   _f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half),
+                                   _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, head_dim,
+                                   _chk(workspace, "workspace", torch.uint8, 1), workspace.numel(), qn,
+                                   int(causal_prefix), _stream())
         _lib.check(rc, "cdm_attn_fwd_bf16")
         return out
-    # timed form: the same two stages, with HIP events around the attention kernel alone
-    rc = lib.cdm_attn_pack_kv_bf16(kp, k.stride(0), vp, v.stride(0), cp, sp, wp, workspace.numel(), n, n_heads,
-                                   head_dim, qn, _stream())
-    _lib.check(rc, "cdm_attn_pack_kv_bf16")
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    rc = lib.cdm_attn_fwd_packed_bf16(qp, q.stride(0), cp, sp, wp, op, out.stride(0), n, n_heads, head_dim, qn, _stream())
-    e1.record()
-    _lib.check(rc, "cdm_attn_fwd_packed_bf16")
-    _ATTN_TIMER.append((e0, e1))
-    return out
+    # two-stage form: prefix images, or HIP events around the attention kernel alone while timing is on
+    attention_pack_kv(k, v, n_heads, head_dim, workspace, cos, sin, qk_norm)
+    return attention_packed(q, workspace, n_heads, head_dim, out, cos, sin, qk_norm, prefix, causal_prefix)
 
 
 def cfg_step(x: torch.Tensor, v_cond: torch.Tensor, v_uncond: Optional[torch.Tensor], guidance: float,

@@ -156,6 +156,9 @@ typedef struct cdm_qk_norm {
  *   q, k, v: [n_tokens, n_heads, head_dim] with row strides ldq, ldk, ldv; o: [n_tokens, n_heads*head_dim] (ldo).
  *   cos, sin: [n_tokens, head_dim/2] fp32 rotary tables, or both null when Q and K are already rotated.
  *   qk_norm: null, or the per-head RMSNorm of Q and K described above.
+ *   causal_prefix: 0 = full attention.  P > 0 = the hybrid mask of the architecture figure
+ *     (cookbooks/cosmos3/cosmos3-model-architecture.png, right panel; README.md:74): the first P tokens (the AR /
+ *     text run) attend causally among themselves and to nothing else, every other token attends to all tokens.
  *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds K and V re-laid
  *   out as 64-key tile images); its contents are undefined afterwards.
  * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
@@ -164,20 +167,26 @@ int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head
 int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
                           const float* cos, const float* sin, void* o, int64_t ldo, int64_t n_tokens,
                           int32_t n_heads, int32_t head_dim, void* workspace, int64_t workspace_bytes,
-                          const cdm_qk_norm* qk_norm, void* stream);
+                          const cdm_qk_norm* qk_norm, int64_t causal_prefix, void* stream);
 
 /*
  * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first K (rotated
  * if tables are given) and V are packed into the workspace as tile images (a streaming pass), then the
  * attention kernel proper reads Q (rotating it with the same tables) and the workspace.  A caller that
  * times or profiles the attention kernel alone, or that reuses packed K/V across calls, uses these.
+ *   prefix_workspace / n_prefix_tokens (optional): tile images, made by an earlier cdm_attn_pack_kv_bf16 call over
+ *   n_prefix_tokens tokens (a multiple of 64), of keys that PRECEDE the keys of `workspace`; the n_tokens queries
+ *   then attend to n_prefix_tokens + n_tokens keys.  Under the hybrid mask the K/V of the text run do not depend on
+ *   the denoising step, so they are packed once per prompt and passed here at every step, and the per-step call
+ *   carries only the generator tokens.  Cannot be combined with causal_prefix.
  */
 int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                               const float* sin, void* workspace, int64_t workspace_bytes, int64_t n_tokens,
                               int32_t n_heads, int32_t head_dim, const cdm_qk_norm* qk_norm, void* stream);
 int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
                                  const void* workspace, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
-                                 int32_t head_dim, const cdm_qk_norm* qk_norm, void* stream);
+                                 int32_t head_dim, const cdm_qk_norm* qk_norm, const void* prefix_workspace,
+                                 int64_t n_prefix_tokens, int64_t causal_prefix, void* stream);
 
 /*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each

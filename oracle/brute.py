@@ -61,12 +61,13 @@ def apply_rope(x, ang):
     return y
 
 
-def attention(q, k, v):
+def attention(q, k, v, kv_end=None):
+    """kv_end[n] (optional): query n sees keys 0 .. kv_end[n]-1 only."""
     N, H, dh = q.shape
-    M = k.shape[0]
     o = np.zeros((N, H, dh))
     for h in range(H):
         for n in range(N):
+            M = k.shape[0] if kv_end is None else int(kv_end[n])
             sc = np.array([sum(q[n, h, c] * k[m, h, c] for c in range(dh)) for m in range(M)]) / math.sqrt(dh)
             e = np.exp(sc - sc.max())
             p = e / e.sum()

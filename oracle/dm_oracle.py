@@ -21,7 +21,7 @@ __all__ = [
     "mrope_axis_map", "text_positions", "vision_positions", "joint_positions",
     "mrope_cos_sin", "apply_mrope", "attention", "attention_rows", "swiglu",
     "dm_block", "dm_stack", "quant_e4m3_rows", "quant_e4m3_weight", "fp8_linear",
-    "max_rel_err", "cos_sim", "E4M3_MAX", "cfg_step", "flow_sigmas",
+    "max_rel_err", "cos_sim", "E4M3_MAX", "cfg_step", "flow_sigmas", "hybrid_kv_end",
 ]
 
 E4M3_MAX = 448.0
@@ -184,30 +184,48 @@ def apply_mrope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.
 # --------------------------------------------------------------------------
 # attention
 # --------------------------------------------------------------------------
-def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+def hybrid_kv_end(n_tokens: int, causal_prefix: int) -> torch.Tensor:
+    """Per-query key limit of the hybrid mask (architecture figure, right panel; REF/README.md:74): the first
+    ``causal_prefix`` tokens (the AR / text run) see keys 0..i (causal, and no generator keys), all later tokens
+    (DM, full attention) see every key.  Query i sees key j iff j < kv_end[i]."""
+    i = torch.arange(n_tokens)
+    return torch.where(i < causal_prefix, i + 1, torch.full_like(i, n_tokens))
+
+
+def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                   kv_end: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Exact attention for a subset of query rows: q_rows[R,H,dh], k,v[N,H,dh] -> [R,H,dh].
 
-    softmax(q k^T / sqrt(dh)) v, fp32 softmax, no mask
+    softmax(q k^T / sqrt(dh)) v, fp32 softmax
     (TF/models/qwen3_vl/modeling_qwen3_vl.py:171-193; non-causal full
-    attention for DM tokens per REF/README.md:74).
+    attention for DM tokens per REF/README.md:74).  ``kv_end[R]``: row r sees
+    keys j < kv_end[r] only (additive -inf mask ahead of the softmax, as the
+    eager form does with its attention_mask, TF/...modeling_qwen3_vl.py:185-186).
     """
     q = q_rows.to(torch.float32).transpose(0, 1).contiguous()   # [H,R,dh]
     kk = k.to(torch.float32).transpose(0, 1).contiguous()       # [H,N,dh]
     vv = v.to(torch.float32).transpose(0, 1).contiguous()
     s = torch.matmul(q, kk.transpose(1, 2)) * (1.0 / math.sqrt(q.shape[-1]))
+    if kv_end is not None:
+        hidden = torch.arange(k.shape[0]).view(1, 1, -1) >= kv_end.view(1, -1, 1)
+        s = s.masked_fill(hidden, float("-inf"))
     p = torch.softmax(s, dim=-1, dtype=torch.float32)
     return torch.matmul(p, vv).transpose(0, 1).contiguous()
 
 
-def attention(q, k, v, chunk: int = 1024) -> torch.Tensor:
-    """Full attention, chunked over query rows so scores are never all resident."""
+def attention(q, k, v, chunk: int = 1024, kv_end: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention, chunked over query rows so scores are never all resident; ``kv_end`` as in attention_rows."""
     kk = k.to(torch.float32).transpose(0, 1).contiguous()
     vv = v.to(torch.float32).transpose(0, 1).contiguous()
     scale = 1.0 / math.sqrt(q.shape[-1])
     out = []
     for i in range(0, q.shape[0], chunk):
         qq = q[i:i + chunk].to(torch.float32).transpose(0, 1).contiguous()
-        p = torch.softmax(torch.matmul(qq, kk.transpose(1, 2)) * scale, dim=-1, dtype=torch.float32)
+        s = torch.matmul(qq, kk.transpose(1, 2)) * scale
+        if kv_end is not None:
+            hidden = torch.arange(k.shape[0]).view(1, 1, -1) >= kv_end[i:i + chunk].view(1, -1, 1)
+            s = s.masked_fill(hidden, float("-inf"))
+        p = torch.softmax(s, dim=-1, dtype=torch.float32)
         out.append(torch.matmul(p, vv).transpose(0, 1))
     return torch.cat(out, 0).contiguous()
 
@@ -261,8 +279,9 @@ def _linear(a, w, fp8):
 def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
              mod: Optional[Sequence[torch.Tensor]], cos: torch.Tensor, sin: torch.Tensor,
              n_heads: int, segments: Optional[Sequence[Segment]] = None, eps: float = 1e-6,
-             fp8: bool = False, attn_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One Mixture-of-Transformers layer over x[N, d].
+             fp8: bool = False, attn_rows: Optional[torch.Tensor] = None, causal_prefix: int = 0) -> torch.Tensor:
+    """One Mixture-of-Transformers layer over x[N, d].  ``causal_prefix`` > 0 selects the hybrid mask
+    (hybrid_kv_end) for the shared attention.
 
     per-branch norm -> per-branch QKV -> mRoPE -> ONE shared full attention
     over all N tokens -> per-branch out-proj, gated residual -> per-branch norm
@@ -294,12 +313,13 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
     q = apply_mrope(q.view(N, n_heads, dh), cos, sin)
     k = apply_mrope(k.view(N, n_heads, dh), cos, sin)
     v = v.view(N, n_heads, dh)
+    kv_end = hybrid_kv_end(N, causal_prefix) if causal_prefix else None
     if attn_rows is None:
-        o = attention(q, k, v).reshape(N, d)
+        o = attention(q, k, v, kv_end=kv_end).reshape(N, d)
         rows = torch.arange(N)
     else:
         rows = attn_rows
-        o = attention_rows(q[rows], k, v).reshape(-1, d)
+        o = attention_rows(q[rows], k, v, kv_end[rows] if kv_end is not None else None).reshape(-1, d)
     xr = x[rows]
     out = torch.empty_like(xr)
     for (s0, ln, ws, modulated) in segments:
@@ -323,10 +343,10 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
 
 def dm_stack(x, blocks: Sequence[Sequence[Dict[str, torch.Tensor]]], mods: Sequence[Optional[Sequence[torch.Tensor]]],
              cos, sin, n_heads: int, segments: Optional[Sequence[Segment]] = None, eps: float = 1e-6,
-             fp8: bool = False) -> torch.Tensor:
+             fp8: bool = False, causal_prefix: int = 0) -> torch.Tensor:
     """L blocks in sequence; ``blocks[l]`` is the list of weight sets of layer l, ``mods[l]`` its modulation."""
     for ws, m in zip(blocks, mods):
-        x = dm_block(x, ws, m, cos, sin, n_heads, segments, eps, fp8)
+        x = dm_block(x, ws, m, cos, sin, n_heads, segments, eps, fp8, causal_prefix=causal_prefix)
     return x
 
 

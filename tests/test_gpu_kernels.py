@@ -233,6 +233,49 @@ def test_attention_with_qk_norm_and_rope(n, H, hd, seg_ends, variant):
     assert_close(o2, o.float().cpu(), 0.9999, 1e-2, "qk-norm scale invariance")
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n,P,H,hd", [(300, 100, 2, 128), (700, 512, 1, 128), (64, 64, 2, 64), (130, 130, 1, 128),
+                                      (577, 1, 1, 64), (900, 256, 1, 128)])
+def test_attention_hybrid_mask(n, P, H, hd, variant):
+    """The first P tokens attend causally among themselves, the others see everything."""
+    g = gen(n + P)
+    d = H * hd
+    qkv, qkvr = rand_bf16((n, 3 * d), g, 1.5)
+    prev = ops.set_variant("attn", variant)
+    try:
+        o = ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], H, hd, causal_prefix=P)
+    finally:
+        ops.set_variant("attn", prev)
+    want = O.attention(qkvr[:, :d].view(n, H, hd), qkvr[:, d:2 * d].view(n, H, hd), qkvr[:, 2 * d:].view(n, H, hd),
+                       kv_end=O.hybrid_kv_end(n, P))
+    assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"hybrid mask n={n} P={P} variant={variant}")
+    assert_close(o[:1], qkvr[:1, 2 * d:], 0.99999, 5e-3, "first token sees only itself")
+
+
+@pytest.mark.parametrize("P,m,H,hd", [(64, 200, 2, 128), (128, 65, 1, 64), (512, 700, 1, 128)])
+def test_attention_with_prefix_key_images(P, m, H, hd):
+    """Keys packed once (the text run) and prepended to the per-call keys: the m query rows must equal rows P.. of
+    full attention over all P + m tokens; mRoPE and QK-norm in registers on both sides."""
+    g = gen(P + m)
+    n, d = P + m, H * hd
+    pos, _ = rotary.build_positions(n, (0, 0, 0), 0)
+    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48) if hd == 128 else (16, 24, 24))
+    cosd, sind = cos.to(dev()), sin.to(dev())
+    qkv, qkvr = rand_bf16((n, 3 * d), g, 1.5)
+    qw, kw = 1 + 0.2 * torch.randn(2, hd, generator=g), 1 + 0.2 * torch.randn(2, hd, generator=g)
+    qwd, kwd = qw.to(dev()), kw.to(dev())
+    k, v, q = qkv[:, d:2 * d], qkv[:, 2 * d:], qkv[:, :d]
+    pre = ops.attention_pack_kv(k[:P], v[:P], H, hd, cos=cosd[:P].contiguous(), sin=sind[:P].contiguous(),
+                                qk_norm=(qwd[:1].contiguous(), kwd[:1].contiguous(), [P], 1e-6))
+    o = ops.attention(q[P:], k[P:], v[P:], H, hd, cos=cosd[P:].contiguous(), sin=sind[P:].contiguous(),
+                      qk_norm=(qwd[1:].contiguous(), kwd[1:].contiguous(), [m], 1e-6), prefix=(pre, P))
+    qn = O.rms_norm(qkvr[:, :d].view(n, H, hd)[P:], qw[1], 1e-6)
+    kn = torch.cat([O.rms_norm(qkvr[:P, d:2 * d].view(P, H, hd), kw[0], 1e-6),
+                    O.rms_norm(qkvr[P:, d:2 * d].view(m, H, hd), kw[1], 1e-6)])
+    want = O.attention(O.apply_mrope(qn, cos[P:], sin[P:]), O.apply_mrope(kn, cos, sin), qkvr[:, 2 * d:].view(n, H, hd))
+    assert_close(o, want.reshape(m, d), 0.9999, 1e-2, f"prefix images P={P} m={m}")
+
+
 def test_attention_closed_forms_and_determinism():
     g = gen(9)
     n, H, hd = 200, 2, 128

@@ -183,3 +183,41 @@ def test_cfg_step_closed_forms():
     assert s1[0] == 1.0 and s1[-1] == 0.0 and torch.allclose(s1, torch.linspace(1, 0, 11, dtype=torch.float64))
     assert s3[0] == 1.0 and s3[-1] == 0.0 and bool((s3[1:] < s3[:-1]).all()) and bool((s3[1:-1] > s1[1:-1]).all())
     assert torch.allclose(s3 * (1 + 2.0 * s1), 3.0 * s1)
+
+
+def test_hybrid_mask_attention():
+    """Masked oracle attention against the float64 brute force (which simply drops the hidden keys) and against
+    the decomposition the mask implies: a prefix row is plain attention over the keys up to itself, a later row is
+    plain attention over everything."""
+    g = torch.Generator().manual_seed(12)
+    N, H, dh, P = 11, 2, 8, 4
+    q, k, v = (torch.randn(N, H, dh, generator=g) for _ in range(3))
+    kv_end = O.hybrid_kv_end(N, P)
+    assert kv_end.tolist() == [1, 2, 3, 4] + [N] * (N - P)
+    got = O.attention(q, k, v, chunk=3, kv_end=kv_end)
+    want = B.attention(q.double().numpy(), k.double().numpy(), v.double().numpy(), kv_end.numpy())
+    assert np.abs(got.double().numpy() - want).max() < 1e-5
+    for i in range(N):
+        e = int(kv_end[i])
+        row = O.attention(q[i:i + 1], k[:e], v[:e])
+        assert torch.allclose(got[i:i + 1], row, atol=1e-6)
+    rows = torch.tensor([0, 3, 4, 10])
+    assert torch.allclose(O.attention_rows(q[rows], k, v, kv_end[rows]), got[rows], atol=1e-6)
+    assert torch.allclose(got[0], v[0], atol=1e-6)            # the first token sees only itself
+    # inside a block: the prefix rows do not depend on anything after the prefix
+    d = H * dh
+    x = torch.randn(N, d, generator=g)
+    w = {n: torch.randn(s, generator=g) * 0.3 for n, s in dict(wq=(d, d), wk=(d, d), wv=(d, d), wo=(d, d), wg=(2 * d, d),
+                                                              wu=(2 * d, d), wd=(d, 2 * d)).items()}
+    w.update(norm1_w=torch.ones(d), norm2_w=torch.ones(d))
+    mod = [torch.randn(d, generator=g) * 0.1 for _ in range(6)]
+    pos = O.text_positions(0, N)
+    cos, sin = O.mrope_cos_sin(pos, dh, (2, 2, 4))
+    segs = [(0, P, 0, False), (P, N - P, 0, True)]
+    y = O.dm_block(x, [w], mod, cos, sin, H, segs, causal_prefix=P)
+    x2 = x.clone(); x2[P:] = torch.randn(N - P, d, generator=g)
+    y2 = O.dm_block(x2, [w], mod, cos, sin, H, segs, causal_prefix=P)
+    assert torch.allclose(y[:P], y2[:P], atol=1e-6) and not torch.allclose(y[P:], y2[P:], atol=1e-3)
+    # ... and equal the block run on the prefix alone with a causal mask
+    y3 = O.dm_block(x[:P], [w], mod, cos[:P], sin[:P], H, [(0, P, 0, False)], causal_prefix=P)
+    assert torch.allclose(y[:P], y3, atol=1e-5)
