@@ -23,6 +23,7 @@ class DMConfig:
     eps: float = 1e-6
     fp8: bool = False
     qk_norm: bool = False                    # per-head RMSNorm of Q and K ahead of the rotation
+    hybrid_mask: bool = False                # text run causal and blind to the generator tokens (else full attention)
     seed: int = 1234
 
     @property

@@ -72,9 +72,13 @@ class DMAttnProcessor:
                  image_rotary_emb: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, *,
                  modality_segments: Optional[Sequence[Segment]] = None, residual: Optional[torch.Tensor] = None,
                  gate: Optional[torch.Tensor] = None, quant_scale: Optional[torch.Tensor] = None,
-                 workspace: Optional[Workspace] = None):
+                 workspace: Optional[Workspace] = None, causal_prefix: int = 0, prefix=None,
+                 kv_images: Optional[torch.Tensor] = None):
+        """``causal_prefix`` = P selects the hybrid mask (the first P tokens, the AR run, causal among themselves and
+        blind to the rest); ``prefix`` = (images, n_tokens) prepends keys packed by an earlier call; ``kv_images``
+        is the buffer this call packs its own K/V into (kept by the caller when it wants to reuse them)."""
         if attention_mask is not None:
-            raise NotImplementedError("the DM branch uses full attention; attention_mask must be None")
+            raise NotImplementedError("masks are selected with causal_prefix; attention_mask must be None")
         if image_rotary_emb is None:
             raise ValueError("image_rotary_emb=(cos, sin) is required")
         batched = hidden_states.dim() == 3
@@ -98,7 +102,8 @@ class DMAttnProcessor:
         qkv = ws.qkv if ws is not None else torch.empty((n, 3 * d), dtype=torch.bfloat16, device=x.device)
         o = ws.attn_out if ws is not None else torch.empty((n, d), dtype=torch.bfloat16, device=x.device)
 
-        wsb = ws.attn_ws if ws is not None else None
+        wsb = kv_images if kv_images is not None else (ws.attn_ws if ws is not None else None)
+        mask_kw = dict(causal_prefix=causal_prefix, prefix=prefix)
         q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
         qkn = attn.qk_norm_args(modality_segments)
         if qkn is not None and self.rope != "in_attention":
@@ -106,15 +111,15 @@ class DMAttnProcessor:
         if self.rope == "gemm_epilogue":
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
                          rope_cols=2 * d, head_dim=attn.head_dim)
-            ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb)
+            ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
         else:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
             if self.rope == "streaming":
                 ops.mrope_qk_(q, k, cos, sin, attn.n_heads, attn.head_dim)
-                ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb)
+                ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
             else:     # in registers, inside the attention kernels
                 ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin,
-                              qk_norm=qkn)
+                              qk_norm=qkn, **mask_kw)
         if attn.fp8:
             oq, so = ops.quant_rows(o)
         else:
@@ -276,7 +281,8 @@ class DMBlock(nn.Module):
     def forward(self, hidden_states: torch.Tensor, temb: torch.Tensor,
                 image_rotary_emb: Tuple[torch.Tensor, torch.Tensor],
                 modality_segments: Optional[Sequence[Segment]] = None, *, inplace: bool = False,
-                modulation: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[Workspace] = None):
+                modulation: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[Workspace] = None,
+                causal_prefix: int = 0, prefix=None, kv_images: Optional[torch.Tensor] = None):
         batched = hidden_states.dim() == 3
         x = _as2d(hidden_states)
         if not inplace:
@@ -292,7 +298,7 @@ class DMBlock(nn.Module):
 
         y, sy = self._norm(x, self.norm1_weight, sh1, sc1, segs, ws.y)
         self.attn(y, image_rotary_emb=image_rotary_emb, modality_segments=segs, residual=x, gate=g1, quant_scale=sy,
-                  workspace=ws)
+                  workspace=ws, causal_prefix=causal_prefix, prefix=prefix, kv_images=kv_images)
         y, sy = self._norm(x, self.norm2_weight, sh2, sc2, segs, ws.y)
         q = self._q if self.fp8 else {}
         _routed_linear(y, sy, self.gate_weight, q.get("gate"), self.up_weight, segs, out=ws.h, epilogue="swiglu",
@@ -328,6 +334,13 @@ class TimestepEmbedder(nn.Module):
         return self.linear_2(torch.nn.functional.silu(self.linear_1(e)))
 
 
+class ContextCache:
+    """Per-layer K/V tile images of the text run (see ``DMStack.precompute_context``)."""
+
+    def __init__(self, images: List[torch.Tensor], n_tokens: int):
+        self.images, self.n_tokens = images, n_tokens
+
+
 class DMStack(nn.Module):
     """L blocks over the joint sequence text | video | action (diffusers transformer forward shape)."""
 
@@ -340,6 +353,8 @@ class DMStack(nn.Module):
                                      for _ in range(cfg.n_blocks)])
         self._rot = None
         self._ws: Optional[Workspace] = None
+        self._rot_gen = None
+        self._ws_gen: Optional[Workspace] = None
 
     @torch.no_grad()
     def reset_parameters(self, seed: Optional[int] = None) -> None:
@@ -373,10 +388,39 @@ class DMStack(nn.Module):
         return self._rot
 
     @torch.no_grad()
+    def precompute_context(self, encoder_hidden_states: torch.Tensor) -> "ContextCache":
+        """Under the hybrid mask the text run never sees a generator token and its branch is not modulated, so its
+        keys and values in every layer depend on the prompt only.  Runs the text run alone (causal) through the stack
+        once and keeps the per-layer K/V tile images; ``forward(..., context_cache=...)`` then carries only the
+        generator tokens at every denoising step."""
+        c = self.cfg
+        if not c.hybrid_mask:
+            raise RuntimeError("context reuse needs the hybrid mask (DMConfig.hybrid_mask)")
+        if c.n_text == 0 or c.n_text % 64:
+            raise ValueError("context reuse needs a text run whose length is a positive multiple of 64")
+        x = _as2d(encoder_hidden_states).clone()
+        if x.shape != (c.n_text, c.d_model):
+            raise ValueError(f"context has shape {tuple(x.shape)}, expected {(c.n_text, c.d_model)}")
+        cos, sin = self.rotary(x.device)
+        rot = (cos[:c.n_text].contiguous(), sin[:c.n_text].contiguous())
+        segs = [(0, c.n_text, 0, False)]
+        ws = Workspace(c.n_text, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
+        nbytes = ops.attn_workspace_bytes(c.n_text, c.n_heads, c.head_dim)
+        images = []
+        for blk in self.blocks:
+            img = torch.empty((nbytes,), dtype=torch.uint8, device=x.device)
+            blk(x, None, rot, segs, inplace=True, workspace=ws, modulation=(None,) * 6, causal_prefix=c.n_text,
+                kv_images=img)
+            images.append(img)
+        return ContextCache(images, c.n_text)
+
+    @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
                 encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
-                return_dict: bool = False):
+                return_dict: bool = False, context_cache: Optional["ContextCache"] = None):
         c = self.cfg
+        if context_cache is not None:
+            return self._forward_cached(hidden_states, timestep, action_states, return_dict, context_cache)
         parts = []
         if c.n_text:
             if encoder_hidden_states is None:
@@ -396,8 +440,38 @@ class DMStack(nn.Module):
         if self._ws is None or not self._ws.fits(c.n_tokens, c.d_model, c.hidden) or self._ws.y.device != x.device:
             self._ws = Workspace(c.n_tokens, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
         for blk in self.blocks:
-            blk(x, temb, rot, segs, inplace=True, workspace=self._ws)
+            blk(x, temb, rot, segs, inplace=True, workspace=self._ws, causal_prefix=c.n_text if c.hybrid_mask else 0)
         video = x[c.n_text:c.n_text + c.n_video]
+        out = video.unsqueeze(0) if hidden_states.dim() == 3 else video
+        if return_dict:
+            return {"sample": out, "joint": x}
+        return (out,)
+
+
+    def _forward_cached(self, hidden_states, timestep, action_states, return_dict, cache: "ContextCache"):
+        c = self.cfg
+        P = c.n_text
+        if cache.n_tokens != P or len(cache.images) != len(self.blocks):
+            raise ValueError("context cache does not belong to this stack")
+        parts = [_as2d(hidden_states)]
+        if c.n_action:
+            if action_states is None:
+                raise ValueError("this configuration expects action_states")
+            parts.append(_as2d(action_states))
+        x = torch.cat(parts, dim=0).contiguous() if len(parts) > 1 else parts[0].clone()
+        n = c.n_tokens - P
+        if x.shape != (n, c.d_model):
+            raise ValueError(f"generator sequence has shape {tuple(x.shape)}, expected {(n, c.d_model)}")
+        if self._rot_gen is None or self._rot_gen[0].device != x.device:
+            cos, sin = self.rotary(x.device)
+            self._rot_gen = (cos[P:].contiguous(), sin[P:].contiguous())
+        segs = [(s0 - P, ln, b, m) for (s0, ln, b, m) in self.segments() if s0 >= P]
+        temb = self.time_embedder(timestep.reshape(-1)[:1])
+        if self._ws_gen is None or not self._ws_gen.fits(n, c.d_model, c.hidden) or self._ws_gen.y.device != x.device:
+            self._ws_gen = Workspace(n, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
+        for blk, img in zip(self.blocks, cache.images):
+            blk(x, temb, self._rot_gen, segs, inplace=True, workspace=self._ws_gen, prefix=(img, P))
+        video = x[:c.n_video]
         out = video.unsqueeze(0) if hidden_states.dim() == 3 else video
         if return_dict:
             return {"sample": out, "joint": x}

@@ -292,3 +292,50 @@ def test_transformer_with_stack_edges_and_loaded_checkpoint(tmp_path):
     assert_close(out["sample"], want, BF16_COS, BF16_REL, "transformer with stack edges")
     want_act = y[12 + cfg.n_video:] @ f(m.action_proj_out.weight).t() + f(m.action_proj_out.bias)
     assert_close(out["action"][0], want_act, BF16_COS, BF16_REL, "action head")
+
+
+def test_hybrid_mask_stack_and_context_reuse():
+    """Two-branch stack under the hybrid mask: (1) joint forward vs the masked fp32 oracle; (2) the text run's K/V
+    packed once per prompt and reused: same video output from a forward that carries only the generator tokens;
+    (3) the reused cache stays valid for another timestep."""
+    cfg = DMConfig("hyb", 256, 2, 128, 512, 2, (2, 5, 8), n_text=64, n_action=7, n_branches=3, qk_norm=True,
+                   hybrid_mask=True)
+    st = DMStack(cfg, device=dev())
+    st.reset_parameters(41)
+    g = torch.Generator(device=dev()).manual_seed(41)
+    with torch.no_grad():
+        for blk in st.blocks:
+            blk.attn.norm_q_weight.copy_(1 + 0.2 * torch.randn(3, 128, generator=g, device=dev()))
+            blk.attn.norm_k_weight.copy_(1 + 0.2 * torch.randn(3, 128, generator=g, device=dev()))
+            blk.adaLN_modulation.bias.copy_(0.2 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
+    gc = torch.Generator().manual_seed(42)
+    xv, xvr = rand_bf16((1, cfg.n_video, 256), gc)
+    xt, xtr = rand_bf16((1, 64, 256), gc)
+    xa, xar = rand_bf16((1, 7, 256), gc)
+    t = torch.tensor([333.0])
+    out = st(xv, t.to(dev()), encoder_hidden_states=xt, action_states=xa, return_dict=True)
+    te = st.time_embedder
+    f = lambda p: p.detach().float().cpu()
+    c = O.time_mlp(O.timestep_embedding(t), f(te.linear_1.weight), f(te.linear_1.bias), f(te.linear_2.weight), f(te.linear_2.bias))
+    mods = [O.adaln_modulation(c, f(b.adaLN_modulation.weight), f(b.adaLN_modulation.bias)) for b in st.blocks]
+    pos = O.joint_positions([("text", 64), ("video", cfg.grid), ("action", 7)])
+    cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+    x0 = torch.cat([xtr[0], xvr[0], xar[0]])
+    want = O.dm_stack(x0, [oracle_weights(b, 3) for b in st.blocks], mods, cos, sin, 2, st.segments(), causal_prefix=64)
+    assert_close(out["joint"], want, BF16_COS, BF16_REL, "hybrid-mask stack (joint)")
+    want_full = O.dm_stack(x0, [oracle_weights(b, 3) for b in st.blocks], mods, cos, sin, 2, st.segments())
+    assert O.max_rel_err(want[:64], want_full[:64]) > 1e-2           # the mask is live
+    # (2) context reuse
+    cache = st.precompute_context(xt)
+    out2 = st(xv, t.to(dev()), action_states=xa, return_dict=True, context_cache=cache)
+    assert_close(out2["sample"][0], out["sample"][0].float().cpu(), 0.99999, 4e-3, "cached context == joint forward")
+    assert_close(out2["sample"][0], want[64:64 + cfg.n_video], BF16_COS, BF16_REL, "cached context vs oracle")
+    # (3) another timestep with the same cache
+    t2 = torch.tensor([871.0])
+    out3 = st(xv, t2.to(dev()), action_states=xa, return_dict=True, context_cache=cache)
+    ref3 = st(xv, t2.to(dev()), encoder_hidden_states=xt, action_states=xa, return_dict=True)
+    assert_close(out3["sample"][0], ref3["sample"][0].float().cpu(), 0.99999, 4e-3, "cache reused at another timestep")
+    # without the hybrid mask the reuse is refused
+    cfg_full = DMConfig("full", 256, 2, 128, 512, 1, (2, 5, 8), n_text=64)
+    with pytest.raises(RuntimeError):
+        DMStack(cfg_full, device=dev()).precompute_context(xt)
