@@ -107,8 +107,8 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-template <int HD, int QS>
-__device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cur, const char* sk_next2,
+template <int HD, int QS, class Mid>
+__device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
                                           f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
@@ -166,6 +166,8 @@ __device__ __forceinline__ void pipe_step(const char* sk_next, const char* sv_cu
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs)
         asm volatile("" : "+v"(pf[qs][0]), "+v"(pf[qs][1]), "+v"(pf[qs][2]), "+v"(pf[qs][3]), "+v"(l_run[qs]));
+    __builtin_amdgcn_sched_barrier(0);
+    mid();                 // the step's synchronisation point for the waves that take it between the two blocks
     __builtin_amdgcn_sched_barrier(0);
     if (next_masked) {     // wave-uniform: before a ragged last tile, and in every step of a causal query block
 #pragma unroll
@@ -409,17 +411,29 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // (s_waitcnt vmcnt(1 tile)): K(j+2) is read at the end of this very step.  After the barrier every wave is
     // done with K(j) and V(j-1), whose slots are refilled with K(j+3) and V(j+2).
     int ks_next = 1, vs_cur = 0;      // ring slots: (j+1)%3 and j%3
+    // Two waves share a SIMD (wave w and w + 4).  Block A of a step is VALU-heavy (exp, pack) and block B is pure
+    // MFMA; if both waves of a SIMD took the step's barrier at the same point they would need the VALU together and
+    // the matrix pipe together.  So the upper four waves take the SAME barrier between block A and block B
+    // instead of in front of block A: they run half a step out of phase, and while one wave of a SIMD is in its
+    // VALU-heavy block the other is in its MFMA block.  Tile lifetimes do not change: a wave still reads K(j+1) and
+    // K(j+2) fragments and V(j) between the barriers that bracket those tiles (K(j+1) has landed one barrier
+    // earlier than the in-phase waves need it).
+    const bool late_sync = QS == 1 && wave >= 4;
 #define CDM_ATTN_STEP(SCUR, SNEXT)                                                                              \
     {                                                                                                           \
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory");                           \
         const int k_fill = vs_cur;                              /* slot of K(j)   == j % 3     */               \
         const int v_fill = ks_next == 2 ? 0 : ks_next + 1;      /* slot of V(j-1) == (j+2) % 3 */               \
-        issue(kbase, kpre, sk_addr, j + 3, k_fill);                                                             \
-        issue(vbase, vpre, sv_addr, j + 2, v_fill);                                                             \
+        auto sync = [&]() {                                                                                     \
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory");                       \
+            issue(kbase, kpre, sk_addr, j + 3, k_fill);                                                         \
+            issue(vbase, vpre, sv_addr, j + 2, v_fill);                                                         \
+        };                                                                                                      \
+        if (!late_sync) sync();                                                                                 \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QS];                                                                                         \
         _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS>(sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,  \
+        pipe_step<HD, QS>([&]() { if (late_sync) sync(); }, sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, \
+                          sk + v_fill * TILE_BYTES, qf, kw,                                                     \
                           SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 == NT), nvalid);  \
         vs_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
