@@ -118,12 +118,14 @@ def main():
         step()
     torch.cuda.synchronize()
     ops.time_attention(True)
+    ops.time_ops(True)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         out = step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     events = ops.time_attention(False)
+    op_events = ops.time_ops(False)
     assert bool(torch.isfinite(out.float()).all()), "non-finite output"
     if args.pmc_copy_mib:
         src = torch.zeros(args.pmc_copy_mib << 18, dtype=torch.int32, device=dev)
@@ -143,6 +145,25 @@ def main():
     gemm_ms_per_block = ms_per_step / cfg.n_blocks - attn_avg_ms     # everything that is not attention
     gemm_tflops = cfg.gemm_flops_per_block() / (gemm_ms_per_block * 1e-3) / 1e12
     peak = PEAK_BF16_TFLOPS
+    # per-category kernel time from HIP events around every launcher (ms per block)
+    cat_ms = {}
+    for cat, a, b in op_events:
+        cat_ms[cat] = cat_ms.get(cat, 0.0) + a.elapsed_time(b)
+    per_block = {k: v / (args.steps * cfg.n_blocks) for k, v in cat_ms.items()}
+    gemm_peak = PEAK_FP8_TFLOPS if cfg.fp8 else peak
+    kernels = {}
+    if per_block.get("gemm"):
+        tf = cfg.gemm_flops_per_block() / (per_block["gemm"] * 1e-3) / 1e12
+        kernels["gemm"] = {"ms_per_block": round(per_block["gemm"], 3), "tflops": round(tf, 1), "frac_of_mfma_peak": round(tf / gemm_peak, 4)}
+    nd = cfg.n_tokens * cfg.d_model
+    hbm_bytes = {"norm": 2 * (3 if cfg.fp8 else 4) * nd,       # two norms per block: read bf16, write bf16 (or e4m3)
+                 "pack_kv": 8 * nd + 8 * cfg.n_tokens * (cfg.head_dim // 2),   # K, V in; two tile images out; cos/sin
+                 "quant": 2 * 3 * nd + 3 * cfg.n_tokens * cfg.hidden,           # attention output and SwiGLU hidden -> e4m3
+                 "rope": 8 * nd}
+    for cat, nbytes in hbm_bytes.items():
+        if per_block.get(cat):
+            gbs = nbytes / (per_block[cat] * 1e-3) / 1e9
+            kernels[cat] = {"ms_per_block": round(per_block[cat], 3), "GBps": round(gbs, 0), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 3)}
     res = {
         "metric": "ms per denoising step (DiT stack) on 1 GPU",
         "value": round(ms_per_step, 2), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -157,6 +178,7 @@ def main():
                      "traffic": ATTN_TRAFFIC_BYTES.get((cfg.n_tokens, cfg.n_heads, cfg.head_dim))
                      if args.attn_variant == 0 else None,
                      "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},
+        "kernels": kernels,
         "extra": {"ms_per_block": round(ms_per_step / cfg.n_blocks, 3),
                   "non_attention_ms_per_block": round(gemm_ms_per_block, 3),
                   "gemm_tflops_lower_bound": round(gemm_tflops, 1),

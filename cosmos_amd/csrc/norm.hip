@@ -71,22 +71,27 @@ __global__ __launch_bounds__(kThreads) void adaln_rmsnorm_kernel(
     }
 
     const float inv_d = 1.0f / (float)d;
-    for (int64_t row = blockIdx.x; row < n_tokens; row += gridDim.x) {
+    // the next row's loads are issued before the current row is reduced, so a workgroup always has a row in flight
+    uint4 raw[MAXC];
+    auto fetch = [&](int64_t row) {
         const uint4* xr = x + row * nchunk;
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+            const int idx = c * kThreads + tid;
+            raw[c] = idx < nchunk ? xr[idx] : make_uint4(0, 0, 0, 0);
+        }
+    };
+    if ((int64_t)blockIdx.x < n_tokens) fetch(blockIdx.x);
+    for (int64_t row = blockIdx.x; row < n_tokens; row += gridDim.x) {
         float xv[MAXC][8];
         float ss = 0.0f;
 #pragma unroll
         for (int c = 0; c < MAXC; ++c) {
-            const int idx = c * kThreads + tid;
-            if (idx < nchunk) {
-                unpack8(xr[idx], xv[c]);
+            unpack8(raw[c], xv[c]);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) ss += xv[c][i] * xv[c][i];
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) xv[c][i] = 0.0f;
-            }
+            for (int i = 0; i < 8; ++i) ss += xv[c][i] * xv[c][i];
         }
+        if (row + gridDim.x < n_tokens) fetch(row + gridDim.x);
         ss = block_reduce<false>(ss, slot_sum, par_sum);
         const float r = rsqrtf(ss * inv_d + eps);
         float amax = 0.0f;

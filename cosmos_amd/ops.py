@@ -45,6 +45,37 @@ def _f32vec(t: Optional[torch.Tensor], name: str, n: int) -> int:
     return _chk(t.reshape(-1), name)
 
 
+_OP_TIMER = None     # None, or the list that collects (category, start event, end event) while timing is on
+
+
+def _timed(category: str):
+    """While ``time_ops(True)`` is in force, bracket every call of the wrapped launcher with a pair of HIP events on
+    the current stream (the stream the kernels are launched on)."""
+    def deco(fn):
+        def wrapper(*args, **kw):
+            rec = _OP_TIMER
+            if rec is None:
+                return fn(*args, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = fn(*args, **kw)
+            e1.record()
+            rec.append((category, e0, e1))
+            return out
+        wrapper.__name__, wrapper.__doc__ = fn.__name__, fn.__doc__
+        return wrapper
+    return deco
+
+
+def time_ops(enable: bool):
+    """Start (True) or stop (False) collecting (category, start, end) HIP event triples around every kernel launcher
+    of this module ("norm", "gemm", "rope", "pack_kv", "quant", "step"; the attention kernel itself is covered by
+    ``time_attention``); stopping returns the list."""
+    global _OP_TIMER
+    prev, _OP_TIMER = _OP_TIMER, ([] if enable else None)
+    return prev
+
+
 def set_variant(op: str, variant: int) -> int:
     lib = _lib.load()
     prev = lib.cdm_set_variant(op.encode(), int(variant))
@@ -54,6 +85,7 @@ def set_variant(op: str, variant: int) -> int:
 
 
 # ----------------------------------------------------------------------------- norm / quant
+@_timed("norm")
 def adaln_rmsnorm(x: torch.Tensor, w: torch.Tensor, shift: Optional[torch.Tensor] = None,
                   scale: Optional[torch.Tensor] = None, eps: float = 1e-6,
                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -72,6 +104,7 @@ def adaln_rmsnorm(x: torch.Tensor, w: torch.Tensor, shift: Optional[torch.Tensor
     return out
 
 
+@_timed("norm")
 def adaln_rmsnorm_quant(x, w, shift=None, scale=None, eps: float = 1e-6, out_q: Optional[torch.Tensor] = None,
                         out_s: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Same norm, output quantised per token to e4m3: returns (yq [n, d] float8_e4m3fn, s_tok [n] fp32)."""
@@ -91,6 +124,7 @@ def adaln_rmsnorm_quant(x, w, shift=None, scale=None, eps: float = 1e-6, out_q: 
     return yq, s
 
 
+@_timed("quant")
 def quant_rows(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-row e4m3 quantisation of a bf16 matrix [rows, cols] (row stride may exceed cols)."""
     lib = _lib.load()
@@ -104,6 +138,7 @@ def quant_rows(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 # ----------------------------------------------------------------------------- GEMM
+@_timed("gemm")
 def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, epilogue: str = "none",
          residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
          cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rope_cols: int = 0,
@@ -131,6 +166,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
     return out
 
 
+@_timed("gemm")
 def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, *,
              w2q: Optional[torch.Tensor] = None, sw2: Optional[torch.Tensor] = None, epilogue: str = "none",
              residual=None, gate=None, cos=None, sin=None, rope_cols: int = 0, head_dim: int = 0,
@@ -154,6 +190,7 @@ def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Ten
     return out
 
 
+@_timed("gemm")
 def grouped_gemm(a: torch.Tensor, ws: Sequence[torch.Tensor], segments: Sequence[Tuple[int, int]], *,
                  w2s: Optional[Sequence[torch.Tensor]] = None, epilogue: str = "none", residual=None,
                  gates: Optional[Sequence[Optional[torch.Tensor]]] = None, cos=None, sin=None, rope_cols: int = 0,
@@ -187,6 +224,7 @@ def grouped_gemm(a: torch.Tensor, ws: Sequence[torch.Tensor], segments: Sequence
 
 
 # ----------------------------------------------------------------------------- RoPE / attention
+@_timed("rope")
 def mrope_qk_(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor, n_heads: int,
               head_dim: int) -> None:
     """In-place rotate-half mRoPE on q and k ([n, n_heads*head_dim] views, any row stride)."""
@@ -215,6 +253,7 @@ def _qk_norm_arg(qk_norm, head_dim: int):
     return C.addressof(st), (st, ends)
 
 
+@_timed("pack_kv")
 def attention_pack_kv(k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
                       workspace: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                       sin: Optional[torch.Tensor] = None, qk_norm=None) -> torch.Tensor:
@@ -288,7 +327,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     need = attn_workspace_bytes(n, n_heads, head_dim)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
-    if _ATTN_TIMER is None and prefix is None:
+    if _ATTN_TIMER is None and _OP_TIMER is None and prefix is None:
         half = head_dim // 2
         qn, _keep = _qk_norm_arg(qk_norm, head_dim)
         rc = lib.cdm_attn_fwd_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _chk(k, "k", torch.bfloat16, 2),
@@ -304,6 +343,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     return attention_packed(q, workspace, n_heads, head_dim, out, cos, sin, qk_norm, prefix, causal_prefix)
 
 
+@_timed("step")
 def cfg_step(x: torch.Tensor, v_cond: torch.Tensor, v_uncond: Optional[torch.Tensor], guidance: float,
              coef: Sequence[float], hist: Sequence[torch.Tensor] = (), v_out: Optional[torch.Tensor] = None,
              out: Optional[torch.Tensor] = None) -> torch.Tensor:
