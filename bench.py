@@ -63,12 +63,52 @@ def cpu_baseline(cfg, sample_tokens: int):
                       f"x{max(cfg.n_blocks, 1)} blocks"}
 
 
+def bench_attention_only(cfg, args, dev):
+    """Workload C1: 3-D mRoPE + full attention alone on the 16x44x80 grid (56,320 tokens, 32 x 128 heads)."""
+    import torch
+    from cosmos_amd import ops, rotary
+    n, H, hd = cfg.n_tokens, cfg.n_heads, cfg.head_dim
+    d = H * hd
+    g = torch.Generator(device=dev).manual_seed(cfg.seed)
+    qkv = (torch.randn((n, 3 * d), generator=g, device=dev) / hd ** 0.5).to(torch.bfloat16)
+    pos, _ = rotary.build_positions(0, cfg.grid, 0)
+    cos, sin = rotary.rotary_tables(pos, hd, cfg.mrope_sections, cfg.rope_base, cfg.rope_layout, dev)
+    out = torch.empty((n, d), dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(ops.attn_workspace_bytes(n, H, hd), dtype=torch.uint8, device=dev)
+    step = lambda: ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], H, hd, out=out, workspace=ws, cos=cos, sin=sin)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ops.time_attention(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev = ops.time_attention(False)
+    assert bool(torch.isfinite(out.float()).all()), "non-finite output"
+    ms = wall * 1e3 / args.steps
+    k_ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
+    flops = 4.0 * float(n) ** 2 * d
+    tf = flops / (k_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "ms per mRoPE + attention pass on 1 GPU", "value": round(ms, 3), "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"C1: mRoPE + full attention, {H}x{hd} heads, grid {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} = {n} tokens",
+                   "n_tokens": n, "attn_variant": args.attn_variant},
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": flops, "avg_launch_ms": round(k_ms, 3), "launches": len(ev)},
+        "extra": {"pack_kv_and_launch_overhead_ms": round(ms - k_ms, 3), "device": torch.cuda.get_device_name(0)}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--workload", default="C2", choices=["C0", "C2", "C3", "C4"])
+    ap.add_argument("--workload", default="C2", choices=["C0", "C1", "C2", "C3", "C4"])
     ap.add_argument("--blocks", type=int, default=0, help="override the number of blocks (measurement aid; 0 = config)")
     ap.add_argument("--attn-variant", type=int, default=0)
     ap.add_argument("--gemm-variant", type=int, default=0)
@@ -96,9 +136,13 @@ def main():
     if args.blocks:
         cfg = dataclasses.replace(cfg, n_blocks=args.blocks)
     _lib.load()
+    if args.workload == "C1" and args.steps == 3:
+        args.steps = 10
     ops.set_variant("attn", args.attn_variant)
     ops.set_variant("gemm", args.gemm_variant)
 
+    if args.workload == "C1":
+        return bench_attention_only(cfg, args, dev)
     stack = DMStack(cfg, device=dev)
     stack.reset_parameters()
     if args.rope != "in_attention":

@@ -339,3 +339,42 @@ def test_hybrid_mask_stack_and_context_reuse():
     cfg_full = DMConfig("full", 256, 2, 128, 512, 1, (2, 5, 8), n_text=64)
     with pytest.raises(RuntimeError):
         DMStack(cfg_full, device=dev()).precompute_context(xt)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_c2_full_size_gemms_sampled_rows(fp8):
+    """The four linear layers of a block at the full C2 / C4 shape (56,832 tokens, d 4096, hidden 16384) on the GPU;
+    512 sampled token rows are recomputed in fp32 on the host (rows of a linear layer are independent, so a row
+    sample is an exact check of those rows), plus linearity in the activation at full size."""
+    N, d, h = 56832, 4096, 16384
+    g = torch.Generator(device=dev()).manual_seed(1236)
+    rnd = lambda *s, sd=1.0: (torch.randn(s, generator=g, device=dev()) * sd).to(torch.bfloat16)
+    x, hid = rnd(N, d), rnd(N, h)
+    wqkv, wo, wg, wu, wd = rnd(3 * d, d, sd=0.02), rnd(d, d, sd=0.02), rnd(h, d, sd=0.02), rnd(h, d, sd=0.02), rnd(d, h, sd=0.02)
+    res = rnd(N, d)
+    gate = torch.randn(d, generator=g, device=dev())
+    rows = torch.randperm(N, generator=torch.Generator().manual_seed(3))[:512].sort().values
+    rd = rows.to(dev())
+    f = lambda t: t.float().cpu()
+    xs, hs, rs = f(x[rd]), f(hid[rd]), f(res[rd])
+    tol = (FP8_COS, FP8_REL) if fp8 else (BF16_COS, 1e-2)
+    if fp8:
+        xq, sx = ops.quant_rows(x); hq, sh = ops.quant_rows(hid)
+        q = {n: ops.quant_rows(w) for n, w in dict(qkv=wqkv, o=wo, g=wg, u=wu, d=wd).items()}
+        qkv = ops.gemm_fp8(xq, sx, *q["qkv"])
+        o = ops.gemm_fp8(xq, sx, *q["o"], epilogue="gate_residual", residual=res, gate=gate)
+        hh = ops.gemm_fp8(xq, sx, *q["g"], w2q=q["u"][0], sw2=q["u"][1], epilogue="swiglu")
+        dn = ops.gemm_fp8(hq, sh, *q["d"], epilogue="gate_residual", residual=res, gate=gate)
+    else:
+        qkv = ops.gemm(x, wqkv)
+        o = ops.gemm(x, wo, epilogue="gate_residual", residual=res, gate=gate)
+        hh = ops.gemm(x, wg, w2=wu, epilogue="swiglu")
+        dn = ops.gemm(hid, wd, epilogue="gate_residual", residual=res, gate=gate)
+    assert_close(qkv[rd], xs @ f(wqkv).t(), *tol, "QKV rows")
+    assert_close(o[rd], rs + f(gate) * (xs @ f(wo).t()), *tol, "out-proj + gated residual rows")
+    assert_close(hh[rd], torch.nn.functional.silu(xs @ f(wg).t()) * (xs @ f(wu).t()), tol[0] - (0.002 if fp8 else 0), tol[1] * (1.6 if fp8 else 1), "SwiGLU rows")
+    assert_close(dn[rd], rs + f(gate) * (hs @ f(wd).t()), *tol, "down-proj + gated residual rows")
+    assert bool(torch.isfinite(qkv.float()).all()) and bool(torch.isfinite(dn.float()).all())
+    if not fp8:
+        # linearity at full size: gemm(2x) == 2 gemm(x) exactly (a power of two commutes with every rounding)
+        assert torch.equal(ops.gemm(x * 2, wo), qkv.new_tensor(2.0) * ops.gemm(x, wo))
