@@ -28,18 +28,73 @@ typedef __attribute__((address_space(3))) void lds_void;
 
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 
+constexpr int kMaxSeg = 8;
+
+// One launch covers up to kMaxSeg contiguous row segments of A / C / R, each with its own weights (the MoT
+// branches): the grid is the concatenation of the segments' tile lists, so the few tiles of a short segment (a
+// 256-token action run, a 512-token text run) fill the tail of the long segment's grid instead of paying for a
+// launch of their own that cannot fill the chip.
+struct GemmSeg {
+    int m_start, m_end;                  // token rows [m_start, m_end)
+    int tiles_m, tile_end;               // row tiles of the segment; tiles of segments 0..this one
+    const void* W; const void* W2;
+    const float* gate;
+    const float* sw; const float* sw2;   // fp8 only
+};
+
 struct GemmParams {
     const void* A; int64_t lda;          // operand strides in BYTES
-    const void* W; const void* W2; int64_t ldw;
-    const float* sa; const float* sw; const float* sw2;   // fp8 only
+    int64_t ldw;
+    const float* sa;                     // fp8 only: per-row scale of A, indexed by the global row
     bf16_t* C; int64_t ldc;
-    int M, N, K;
+    int N, K;
     const bf16_t* R; int64_t ldr;
-    const float* gate;
     const float* cos; const float* sin;
     int rope_cols, head_dim;
-    int tiles_m, tiles_n;
+    int tiles_n, total_tiles, n_seg;
+    GemmSeg seg[kMaxSeg];
 };
+
+// what a workgroup works on
+struct Tile {
+    int m0, m_end, tn;
+    const void* W; const void* W2;
+    const float* gate; const float* sw; const float* sw2;
+};
+
+// XCD-aware tile assignment: workgroup ids are dealt round-robin over the 8 XCDs, so ids are remapped to give each
+// XCD a contiguous range of tiles; inside a segment, tiles are ordered in groups of 8 row tiles x all column tiles,
+// column-major inside the group, so that the 32 tiles an XCD runs at a time share 8 A slabs and 4 W slabs in its L2.
+template <class T>
+__device__ __forceinline__ T* uniform_ptr(T* ptr) {      // wave-uniform value -> scalar registers
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
+    const int per_xcd = (p.total_tiles + 7) >> 3;
+    int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.total_tiles) return false;
+    int si = 0;
+#pragma unroll
+    for (int i = 0; i < kMaxSeg - 1; ++i) si += (i < p.n_seg - 1 && logical >= p.seg[i].tile_end) ? 1 : 0;
+    const GemmSeg& sg = p.seg[si];
+    logical -= si ? p.seg[si - 1].tile_end : 0;
+    constexpr int GM = 8;
+    const int group = logical / (GM * p.tiles_n);
+    const int first_m = group * GM;
+    const int gsz = (sg.tiles_m - first_m) < GM ? (sg.tiles_m - first_m) : GM;
+    const int in_group = logical - group * GM * p.tiles_n;
+    // everything here is a function of blockIdx: pin it to scalar registers (the segment table is indexed
+    // dynamically, which the compiler would otherwise treat as a per-lane value)
+    t.m0 = __builtin_amdgcn_readfirstlane(sg.m_start + (first_m + in_group % gsz) * BM);
+    t.m_end = __builtin_amdgcn_readfirstlane(sg.m_end);
+    t.tn = __builtin_amdgcn_readfirstlane(in_group / gsz);
+    t.W = uniform_ptr(sg.W); t.W2 = uniform_ptr(sg.W2);
+    t.gate = uniform_ptr(sg.gate); t.sw = uniform_ptr(sg.sw); t.sw2 = uniform_ptr(sg.sw2);
+    return true;
+}
 
 // chunk swizzle: 16-byte chunk c of tile row r lives at chunk position c ^ swz(r)
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
@@ -122,8 +177,8 @@ __device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) 
 }
 
 template <int EPI, bool FP8>
-__device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4], int m0, int n0, int wm, int wn,
-                                         int lane) {
+__device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32x16 (&acc)[4][4], int m0, int n0, int wm,
+                                         int wn, int lane) {
     const int r32 = lane & 31, kh = lane >> 5;
     const int row_base = m0 + wm * 128 + r32;
     if (EPI == CDM_EPI_SWIGLU) {
@@ -131,7 +186,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             const int row = row_base + mi * 32;
-            if (row >= p.M) continue;
+            if (row >= t.m_end) continue;
             const float sr = FP8 ? p.sa[row] : 1.0f;
             bf16_t* crow = p.C + (int64_t)row * p.ldc;
 #pragma unroll
@@ -142,8 +197,8 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4
                     if (col >= p.N) continue;
                     float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
                     if (FP8) {
-                        const float4 a = *reinterpret_cast<const float4*>(p.sw + col);
-                        const float4 b = *reinterpret_cast<const float4*>(p.sw2 + col);
+                        const float4 a = *reinterpret_cast<const float4*>(t.sw + col);
+                        const float4 b = *reinterpret_cast<const float4*>(t.sw2 + col);
                         sg[0] = a.x * sr; sg[1] = a.y * sr; sg[2] = a.z * sr; sg[3] = a.w * sr;
                         su[0] = b.x * sr; su[1] = b.y * sr; su[2] = b.z * sr; su[3] = b.w * sr;
                     }
@@ -162,7 +217,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
         const int row = row_base + mi * 32;
-        if (row >= p.M) continue;
+        if (row >= t.m_end) continue;
         if (FP8) {      // rank-1 dequantisation scale on the fp32 accumulators
             const float sr = p.sa[row];
 #pragma unroll
@@ -170,7 +225,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int col = col_base + ni * 32 + 8 * g;
-                    const float4 w4 = col < p.N ? *reinterpret_cast<const float4*>(p.sw + col) : make_float4(0, 0, 0, 0);
+                    const float4 w4 = col < p.N ? *reinterpret_cast<const float4*>(t.sw + col) : make_float4(0, 0, 0, 0);
                     acc[mi][ni][4 * g + 0] *= sr * w4.x;
                     acc[mi][ni][4 * g + 1] *= sr * w4.y;
                     acc[mi][ni][4 * g + 2] *= sr * w4.z;
@@ -211,7 +266,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, f32x16 (&acc)[4][4
                 if (EPI == CDM_EPI_GATE_RESIDUAL) {
                     const uint2 r2 = *reinterpret_cast<const uint2*>(rrow + col);
                     float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
-                    if (p.gate) g4 = *reinterpret_cast<const float4*>(p.gate + col);
+                    if (t.gate) g4 = *reinterpret_cast<const float4*>(t.gate + col);
                     o[0] = bf16lo(r2.x) + g4.x * o[0];
                     o[1] = bf16hi(r2.x) + g4.y * o[1];
                     o[2] = bf16lo(r2.y) + g4.z * o[2];
@@ -229,23 +284,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     __shared__ __attribute__((aligned(1024))) char sa1[kTileBytes];
     __shared__ __attribute__((aligned(1024))) char sb1[kTileBytes];
 
-    // ---- XCD-aware tile assignment
-    const int total = p.tiles_m * p.tiles_n;
-    const int per_xcd = (total + 7) >> 3;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
-    constexpr int GM = 8;
-    const int group = logical / (GM * p.tiles_n);
-    const int first_m = group * GM;
-    const int gsz = (p.tiles_m - first_m) < GM ? (p.tiles_m - first_m) : GM;
-    const int in_group = logical - group * GM * p.tiles_n;
-    const int tm = first_m + in_group % gsz;
-    const int tn = in_group / gsz;
+    Tile tile;
+    if (!locate_tile(p, tile)) return;
+    const int tn = tile.tn;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = tm * BM;
+    const int m0 = tile.m0;
     const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
 
     // ---- per-lane byte offsets (relative to the tile's first row) of the 8 + 8 loads of one k-tile
@@ -257,7 +303,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         const int row = (i * 4 + wave) * 8 + (lane >> 3);   // tile row this lane feeds
         const int chunk = (lane & 7) ^ swz(row);            // source chunk that belongs at position lane&7
         int am = row;
-        am = (m0 + am) < p.M ? am : p.M - 1 - m0;
+        am = (m0 + am) < tile.m_end ? am : tile.m_end - 1 - m0;
         oa[i] = (uint32_t)(am * (int)p.lda + chunk * 16);
         int bn;
         if (EPI == CDM_EPI_SWIGLU) {
@@ -272,8 +318,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         ob[i] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
     }
     const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
-    const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)nb0 * p.ldw;
-    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)nb0 * p.ldw : wbase;
+    const char* wbase = reinterpret_cast<const char*>(tile.W) + (int64_t)nb0 * p.ldw;
+    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(tile.W2) + (int64_t)nb0 * p.ldw : wbase;
 
     f32x16 acc[4][4];
 #pragma unroll
@@ -301,7 +347,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         compute_stage<FP8>(sa1, sb1, acc, wm, wn, lane);
     }
 
-    epilogue<EPI, FP8>(p, acc, m0, n0, wm, wn, lane);
+    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -343,22 +389,14 @@ template <int EPI, bool FP8>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_ring_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(1024))) char s_ring[5 * kGranule];
 
-    const int total = p.tiles_m * p.tiles_n;
-    const int per_xcd = (total + 7) >> 3;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
-    constexpr int GM = 8;
-    const int group = logical / (GM * p.tiles_n);
-    const int first_m = group * GM;
-    const int gsz = (p.tiles_m - first_m) < GM ? (p.tiles_m - first_m) : GM;
-    const int in_group = logical - group * GM * p.tiles_n;
-    const int tm = first_m + in_group % gsz;
-    const int tn = in_group / gsz;
+    Tile tile;
+    if (!locate_tile(p, tile)) return;
+    const int tn = tile.tn;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = tm * BM;
+    const int m0 = tile.m0;
     const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
 
     // per-lane byte offsets of the 8 + 8 loads of one k-tile (each instruction = 8 tile rows of 128 bytes)
@@ -368,7 +406,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         const int row = (j * 4 + wave) * 8 + (lane >> 3);
         const int chunk = (lane & 7) ^ swz128(row);
         int am = row;
-        am = (m0 + am) < p.M ? am : p.M - 1 - m0;
+        am = (m0 + am) < tile.m_end ? am : tile.m_end - 1 - m0;
         oa[j] = (uint32_t)(am * (int)p.lda + chunk * 16);
         // SWIGLU: tile rows come in 64-row groups [gate | up | gate | up]; the rows of load j lie in group j / 2
         int bn = (EPI == CDM_EPI_SWIGLU) ? (j >> 2) * 64 + (row & 63) : row;
@@ -376,8 +414,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         ob[j] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
     }
     const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
-    const char* wbase = reinterpret_cast<const char*>(p.W) + (int64_t)n0 * p.ldw;
-    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(p.W2) + (int64_t)n0 * p.ldw : wbase;
+    const char* wbase = reinterpret_cast<const char*>(tile.W) + (int64_t)n0 * p.ldw;
+    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(tile.W2) + (int64_t)n0 * p.ldw : wbase;
     const uint32_t l0 = lds_addr_of(s_ring) + wave * 1024;
 
     f32x16 acc[4][4];
@@ -485,7 +523,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #undef CDM_KSTEP
 #undef CDM_FENCE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // surplus loads must not outlive the workgroup's LDS
-    epilogue<EPI, FP8>(p, acc, m0, n0, wm, wn, lane);
+    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane);
 }
 
 // esize = bytes per operand element (2 = bf16, 1 = e4m3); strides in elements
@@ -527,26 +565,98 @@ int32_t validate(const char* who, int esize, const void* A, int64_t lda, const v
     return CDM_OK;
 }
 
+// host-side description of one row segment of a (grouped) GEMM
+struct HostSeg {
+    int64_t start, len;
+    const void* W; const void* W2;
+    const float* gate; const float* sw; const float* sw2;
+};
+
+// Launches the segments kMaxSeg at a time (one grid per batch).  p holds everything that is common to the segments.
 template <bool FP8>
-int32_t run(GemmParams& p, int64_t M, int64_t N, int32_t epilogue, hipStream_t st, const char* who) {
-    p.tiles_m = (int)((M + BM - 1) / BM);
+int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epilogue, hipStream_t st, const char* who) {
     const int tile_n = epilogue == CDM_EPI_SWIGLU ? BN / 2 : BN;
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
-    const int total = p.tiles_m * p.tiles_n;
-    const int grid = ((total + 7) / 8) * 8;
     // variant 0 = ring pipeline (default); 1 = two-stage pipeline
     const bool ring = cdm_get_variant(1) != 1;
+    int i = 0;
+    while (i < n_seg) {
+        int ns = 0, total = 0;
+        for (; i < n_seg && ns < kMaxSeg; ++i) {
+            if (segs[i].len == 0) continue;
+            GemmSeg& g = p.seg[ns++];
+            g.m_start = (int)segs[i].start; g.m_end = (int)(segs[i].start + segs[i].len);
+            g.tiles_m = (int)((segs[i].len + BM - 1) / BM);
+            total += g.tiles_m * p.tiles_n;
+            g.tile_end = total;
+            g.W = segs[i].W; g.W2 = segs[i].W2; g.gate = segs[i].gate; g.sw = segs[i].sw; g.sw2 = segs[i].sw2;
+        }
+        if (ns == 0) break;
+        p.n_seg = ns; p.total_tiles = total;
+        const int grid = ((total + 7) / 8) * 8;
 #define CDM_LAUNCH(E)                                                         \
     if (ring) gemm_ring_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p);         \
     else gemm_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p)
-    switch (epilogue) {
-        case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;
-        case CDM_EPI_SWIGLU: CDM_LAUNCH(CDM_EPI_SWIGLU); break;
-        case CDM_EPI_GATE_RESIDUAL: CDM_LAUNCH(CDM_EPI_GATE_RESIDUAL); break;
-        default: CDM_LAUNCH(CDM_EPI_ROPE_QK); break;
-    }
+        switch (epilogue) {
+            case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;
+            case CDM_EPI_SWIGLU: CDM_LAUNCH(CDM_EPI_SWIGLU); break;
+            case CDM_EPI_GATE_RESIDUAL: CDM_LAUNCH(CDM_EPI_GATE_RESIDUAL); break;
+            default: CDM_LAUNCH(CDM_EPI_ROPE_QK); break;
+        }
 #undef CDM_LAUNCH
-    return cdm_check_launch(who);
+        int32_t rc = cdm_check_launch(who);
+        if (rc) return rc;
+    }
+    return CDM_OK;
+}
+
+// validates every segment of a grouped call (before anything is enqueued) and fills the host segment list
+template <bool FP8>
+int32_t grouped(const char* who, const void* A, int64_t lda, const float* sa, const void* const* W, const float* const* sw,
+                int64_t ldw, const void* const* W2, const float* const* sw2, void* C, int64_t ldc,
+                const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg, int64_t N, int64_t K, int32_t epilogue,
+                const void* R, int64_t ldr, const float* const* gate, const float* cos, const float* sin,
+                int64_t rope_cols, int32_t head_dim, void* stream) {
+    constexpr int esize = FP8 ? 1 : 2;
+    CDM_REQUIRE(A && W && C && seg_start && seg_len, CDM_ERR_BAD_ARG, "%s: null pointer", who);
+    CDM_REQUIRE(n_seg >= 0 && n_seg <= 64, CDM_ERR_BAD_ARG, "%s: n_seg=%d out of range", who, n_seg);
+    if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(W2, CDM_ERR_BAD_ARG, "%s: SWIGLU needs W2", who);
+    if (FP8) {
+        CDM_REQUIRE(sa && sw, CDM_ERR_BAD_ARG, "%s: null scale pointer", who);
+        if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(sw2, CDM_ERR_BAD_ARG, "%s: SWIGLU needs sw2", who);
+    }
+    HostSeg segs[64];
+    int64_t max_end = 0;
+    for (int g = 0; g < n_seg; ++g) {
+        CDM_REQUIRE(seg_start[g] >= 0 && seg_len[g] >= 0, CDM_ERR_BAD_ARG, "%s: negative segment", who);
+        CDM_REQUIRE(W[g], CDM_ERR_BAD_ARG, "%s: null weight for segment %d", who, g);
+        int32_t rc = validate(who, esize, A, lda, W[g], ldw, W2 ? W2[g] : nullptr, C, ldc, seg_len[g], N, K, epilogue, R, ldr,
+                              cos, sin, rope_cols, head_dim);
+        if (rc) return rc;
+        const float* gt = gate ? gate[g] : nullptr;
+        CDM_REQUIRE(cdm_aligned16(gt), CDM_ERR_BAD_ALIGN, "%s: gate of segment %d must be 16-byte aligned", who, g);
+        if (FP8) {
+            CDM_REQUIRE(sw[g] && cdm_aligned16(sw[g]) && (epilogue != CDM_EPI_SWIGLU || (sw2[g] && cdm_aligned16(sw2[g]))),
+                        CDM_ERR_BAD_ARG, "%s: weight scales of segment %d null or misaligned", who, g);
+        }
+        for (int h = 0; h < g; ++h)
+            CDM_REQUIRE(seg_start[g] >= segs[h].start + segs[h].len || seg_start[g] + seg_len[g] <= segs[h].start,
+                        CDM_ERR_BAD_ARG, "%s: segments %d and %d overlap", who, h, g);
+        segs[g] = HostSeg{seg_start[g], seg_len[g], W[g], W2 ? W2[g] : nullptr, gt, FP8 ? sw[g] : nullptr,
+                          (FP8 && sw2) ? sw2[g] : nullptr};
+        if (seg_start[g] + seg_len[g] > max_end) max_end = seg_start[g] + seg_len[g];
+    }
+    CDM_REQUIRE(max_end < (1ll << 31) - 512, CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
+    if (max_end == 0) return CDM_OK;
+    int32_t rc = cdm_require_device();
+    if (rc) return rc;
+    GemmParams p{};
+    p.A = A; p.lda = lda * esize; p.ldw = ldw * esize; p.sa = sa;
+    p.C = (bf16_t*)C; p.ldc = ldc;
+    p.N = (int)N; p.K = (int)K;
+    p.R = (const bf16_t*)R; p.ldr = ldr;
+    p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
+    return run<FP8>(p, segs, n_seg, N, epilogue, (hipStream_t)stream, who);
 }
 
 }  // namespace
@@ -555,20 +665,10 @@ extern "C" int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int6
                                  int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epilogue, const void* R,
                                  int64_t ldr, const float* gate, const float* cos, const float* sin,
                                  int64_t rope_cols, int32_t head_dim, void* stream) {
-    int32_t rc = validate("gemm_bf16", 2, A, lda, W, ldw, W2, C, ldc, M, N, K, epilogue, R, ldr, cos, sin, rope_cols,
-                          head_dim);
-    if (rc) return rc;
-    CDM_REQUIRE(cdm_aligned16(gate), CDM_ERR_BAD_ALIGN, "gemm_bf16: gate must be 16-byte aligned");
-    if ((rc = cdm_require_device())) return rc;
-    if (M == 0) return CDM_OK;
-    GemmParams p{};
-    p.A = A; p.lda = lda * 2;
-    p.W = W; p.W2 = W2; p.ldw = ldw * 2;
-    p.C = (bf16_t*)C; p.ldc = ldc;
-    p.M = (int)M; p.N = (int)N; p.K = (int)K;
-    p.R = (const bf16_t*)R; p.ldr = ldr; p.gate = gate;
-    p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
-    return run<false>(p, M, N, epilogue, (hipStream_t)stream, "gemm_bf16");
+    const int64_t start = 0;
+    const void* w2[1] = {W2};
+    return grouped<false>("gemm_bf16", A, lda, nullptr, &W, nullptr, ldw, W2 ? w2 : nullptr, nullptr, C, ldc, &start, &M, 1, N,
+                          K, epilogue, R, ldr, &gate, cos, sin, rope_cols, head_dim, stream);
 }
 
 extern "C" int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const void* Wq, int64_t ldw,
@@ -576,24 +676,12 @@ extern "C" int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, co
                                 int64_t N, int64_t K, int32_t epilogue, const void* R, int64_t ldr, const float* gate,
                                 const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
                                 void* stream) {
-    int32_t rc = validate("gemm_fp8", 1, Aq, lda, Wq, ldw, W2q, C, ldc, M, N, K, epilogue, R, ldr, cos, sin, rope_cols,
-                          head_dim);
-    if (rc) return rc;
+    const int64_t start = 0;
+    const void* w2[1] = {W2q};
+    const float* s2[1] = {sw2};
     CDM_REQUIRE(sa && sw, CDM_ERR_BAD_ARG, "gemm_fp8: null scale pointer");
-    if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(sw2, CDM_ERR_BAD_ARG, "gemm_fp8: SWIGLU needs sw2");
-    CDM_REQUIRE(cdm_aligned16(gate) && cdm_aligned16(sw) && cdm_aligned16(sw2), CDM_ERR_BAD_ALIGN,
-                "gemm_fp8: gate and weight-scale vectors must be 16-byte aligned");
-    if ((rc = cdm_require_device())) return rc;
-    if (M == 0) return CDM_OK;
-    GemmParams p{};
-    p.A = Aq; p.lda = lda;
-    p.W = Wq; p.W2 = W2q; p.ldw = ldw;
-    p.sa = sa; p.sw = sw; p.sw2 = sw2;
-    p.C = (bf16_t*)C; p.ldc = ldc;
-    p.M = (int)M; p.N = (int)N; p.K = (int)K;
-    p.R = (const bf16_t*)R; p.ldr = ldr; p.gate = gate;
-    p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
-    return run<true>(p, M, N, epilogue, (hipStream_t)stream, "gemm_fp8");
+    return grouped<true>("gemm_fp8", Aq, lda, sa, &Wq, &sw, ldw, W2q ? w2 : nullptr, s2, C, ldc, &start, &M, 1, N, K, epilogue,
+                         R, ldr, &gate, cos, sin, rope_cols, head_dim, stream);
 }
 
 extern "C" int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw,
@@ -602,30 +690,16 @@ extern "C" int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void*
                                          int32_t epilogue, const void* R, int64_t ldr, const float* const* gate,
                                          const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
                                          void* stream) {
-    CDM_REQUIRE(A && W && C && seg_start && seg_len, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: null pointer");
-    CDM_REQUIRE(n_seg >= 0 && n_seg <= 64, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: n_seg=%d out of range", n_seg);
-    if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(W2, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: SWIGLU needs W2");
-    // validate every segment before anything is enqueued
-    for (int g = 0; g < n_seg; ++g) {
-        CDM_REQUIRE(seg_start[g] >= 0 && seg_len[g] >= 0, CDM_ERR_BAD_ARG, "grouped_gemm_bf16: negative segment");
-        CDM_REQUIRE(W[g], CDM_ERR_BAD_ARG, "grouped_gemm_bf16: null weight for segment %d", g);
-        CDM_REQUIRE((seg_start[g] * lda) % 8 == 0 && (seg_start[g] * ldc) % 8 == 0, CDM_ERR_BAD_ALIGN,
-                    "grouped_gemm_bf16: segment %d does not start on a 16-byte boundary", g);
-        const bf16_t* a = (const bf16_t*)A + seg_start[g] * lda;
-        int32_t rc = validate("grouped_gemm_bf16", 2, a, lda, W[g], ldw, W2 ? W2[g] : nullptr,
-                              (bf16_t*)C + seg_start[g] * ldc, ldc, seg_len[g], N, K, epilogue,
-                              R ? (const bf16_t*)R + seg_start[g] * ldr : nullptr, ldr, cos, sin, rope_cols, head_dim);
-        if (rc) return rc;
-    }
-    for (int g = 0; g < n_seg; ++g) {
-        const int64_t s0 = seg_start[g];
-        const int half = head_dim / 2;
-        int32_t rc = cdm_gemm_bf16((const bf16_t*)A + s0 * lda, lda, W[g], ldw, W2 ? W2[g] : nullptr,
-                                   (bf16_t*)C + s0 * ldc, ldc, seg_len[g], N, K, epilogue,
-                                   R ? (const bf16_t*)R + s0 * ldr : nullptr, ldr, gate ? gate[g] : nullptr,
-                                   cos ? cos + s0 * half : nullptr, sin ? sin + s0 * half : nullptr, rope_cols,
-                                   head_dim, stream);
-        if (rc) return rc;
-    }
-    return CDM_OK;
+    return grouped<false>("grouped_gemm_bf16", A, lda, nullptr, W, nullptr, ldw, W2, nullptr, C, ldc, seg_start, seg_len, n_seg,
+                          N, K, epilogue, R, ldr, gate, cos, sin, rope_cols, head_dim, stream);
+}
+
+extern "C" int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const void* const* Wq,
+                                        const float* const* sw, int64_t ldw, const void* const* W2q,
+                                        const float* const* sw2, void* C, int64_t ldc, const int64_t* seg_start,
+                                        const int64_t* seg_len, int32_t n_seg, int64_t N, int64_t K, int32_t epilogue,
+                                        const void* R, int64_t ldr, const float* const* gate, const float* cos,
+                                        const float* sin, int64_t rope_cols, int32_t head_dim, void* stream) {
+    return grouped<true>("grouped_gemm_fp8", Aq, lda, sa, Wq, sw, ldw, W2q, sw2, C, ldc, seg_start, seg_len, n_seg, N, K,
+                         epilogue, R, ldr, gate, cos, sin, rope_cols, head_dim, stream);
 }

@@ -201,24 +201,27 @@ class DMAttention(nn.Module):
 
 def _routed_linear(a, sa, weights, qweights, weights2, segments, *, out, epilogue, residual=None, gates=None, cos=None,
                    sin=None, rope_cols=0, head_dim=0, qweights2=None) -> None:
-    """Per-modality linear over contiguous token segments (one kernel launch per segment)."""
-    if qweights is None and len(segments) > 1:
-        ops.grouped_gemm(a, [weights[b] for (_, _, b, _) in segments], [(s, l) for (s, l, _, _) in segments],
+    """Per-modality linear over contiguous token segments: one grouped launch over all segments."""
+    segl = [(s, l) for (s, l, _, _) in segments]
+    if qweights is None:
+        if len(segments) == 1:
+            (s0, ln, b, _), = segments
+            sl = slice(s0, s0 + ln)
+            ops.gemm(a[sl], weights[b], w2=weights2[b] if weights2 is not None else None, epilogue=epilogue,
+                     residual=residual[sl] if residual is not None else None, gate=gates[0] if gates is not None else None,
+                     cos=cos[sl] if cos is not None else None, sin=sin[sl] if sin is not None else None,
+                     rope_cols=rope_cols, head_dim=head_dim, out=out[sl])
+            return
+        ops.grouped_gemm(a, [weights[b] for (_, _, b, _) in segments], segl,
                          w2s=[weights2[b] for (_, _, b, _) in segments] if weights2 is not None else None,
                          epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
                          head_dim=head_dim, out=out)
         return
-    for i, (s0, ln, b, _) in enumerate(segments):
-        sl = slice(s0, s0 + ln)
-        kw = dict(epilogue=epilogue, residual=residual[sl] if residual is not None else None,
-                  gate=gates[i] if gates is not None else None, cos=cos[sl] if cos is not None else None,
-                  sin=sin[sl] if sin is not None else None, rope_cols=rope_cols, head_dim=head_dim, out=out[sl])
-        if qweights is not None:
-            wq, sw = qweights[b]
-            w2q, sw2 = qweights2[b] if qweights2 is not None else (None, None)
-            ops.gemm_fp8(a[sl], sa[sl], wq, sw, w2q=w2q, sw2=sw2, **kw)
-        else:
-            ops.gemm(a[sl], weights[b], w2=weights2[b] if weights2 is not None else None, **kw)
+    ops.grouped_gemm_fp8(a, sa, [qweights[b][0] for (_, _, b, _) in segments], [qweights[b][1] for (_, _, b, _) in segments],
+                         segl, w2qs=[qweights2[b][0] for (_, _, b, _) in segments] if qweights2 is not None else None,
+                         sw2s=[qweights2[b][1] for (_, _, b, _) in segments] if qweights2 is not None else None,
+                         epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
+                         head_dim=head_dim, out=out)
 
 
 class DMBlock(nn.Module):

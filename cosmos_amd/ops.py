@@ -223,6 +223,42 @@ def grouped_gemm(a: torch.Tensor, ws: Sequence[torch.Tensor], segments: Sequence
     return out
 
 
+@_timed("gemm")
+def grouped_gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wqs: Sequence[torch.Tensor], sws: Sequence[torch.Tensor],
+                     segments: Sequence[Tuple[int, int]], *, w2qs: Optional[Sequence[torch.Tensor]] = None,
+                     sw2s: Optional[Sequence[torch.Tensor]] = None, epilogue: str = "none", residual=None,
+                     gates: Optional[Sequence[Optional[torch.Tensor]]] = None, cos=None, sin=None, rope_cols: int = 0,
+                     head_dim: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """e4m3 form of ``grouped_gemm``: ``sa`` [M] per-token scales, ``sws[g]`` / ``sw2s[g]`` per-channel weight scales."""
+    lib = _lib.load()
+    M, K = aq.shape
+    N = wqs[0].shape[0]
+    n_seg = len(segments)
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=aq.device)
+    ldw = wqs[0].stride(0)
+    for w in list(wqs) + list(w2qs or []):
+        if w.shape != wqs[0].shape or w.stride(0) != ldw:
+            raise ValueError("all segment weights must share shape and row stride")
+    PP = C.c_void_p * n_seg
+    wp = PP(*[_chk(w, "wq", FP8_DTYPE, 2) for w in wqs])
+    swp = PP(*[_f32vec(s, "sw", N) for s in sws])
+    w2p = PP(*[_chk(w, "w2q", FP8_DTYPE, 2) for w in w2qs]) if w2qs is not None else None
+    sw2p = PP(*[_f32vec(s, "sw2", N) for s in sw2s]) if sw2s is not None else None
+    gp = PP(*[(_f32vec(g, "gate", N) or None) for g in gates]) if gates is not None else None
+    I64 = C.c_int64 * n_seg
+    st, ln = I64(*[int(s) for s, _ in segments]), I64(*[int(l) for _, l in segments])
+    half = head_dim // 2 if head_dim else 0
+    rc = lib.cdm_grouped_gemm_fp8(_chk(aq, "aq", FP8_DTYPE, 2), aq.stride(0), _f32vec(sa, "sa", M), wp, swp, ldw, w2p, sw2p,
+                                  _chk(out, "out", torch.bfloat16, 2), out.stride(0), st, ln, n_seg, N, K,
+                                  _EPI[epilogue], _chk(residual, "residual", torch.bfloat16, 2),
+                                  residual.stride(0) if residual is not None else 0, gp,
+                                  _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols),
+                                  int(head_dim), _stream())
+    _lib.check(rc, "cdm_grouped_gemm_fp8")
+    return out
+
+
 # ----------------------------------------------------------------------------- RoPE / attention
 @_timed("rope")
 def mrope_qk_(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor, n_heads: int,

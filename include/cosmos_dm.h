@@ -193,7 +193,9 @@ int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, c
  * (README.md:53,74 - per-modality weights around one shared attention).  Equivalent to
  * cdm_gemm_bf16 on rows [seg_start[g], seg_start[g] + seg_len[g]) with W[g] (and W2[g], gate[g]).
  * seg_* are HOST arrays of n_seg entries; W/W2/gate are HOST arrays of n_seg device pointers
- * (gate[g] may be null = ungated branch).
+ * (gate[g] may be null = ungated branch).  Segments must not overlap.  All segments run in ONE grid (eight
+ * segments per launch): the tiles of a short segment fill the tail of a long segment's grid.
+ * A, C, R, cos, sin are the tensors of the whole sequence (rows are addressed by their global index).
  */
 int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw,
                               const void* const* W2, void* C, int64_t ldc,
@@ -202,6 +204,17 @@ int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, 
                               const void* R, int64_t ldr, const float* const* gate,
                               const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
                               void* stream);
+
+/* The same for e4m3 operands (see cdm_gemm_fp8): sa is the per-token scale of the whole sequence, sw[g] / sw2[g] the
+ * per-output-channel scales of segment g's weights. */
+int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const void* const* Wq,
+                             const float* const* sw, int64_t ldw, const void* const* W2q,
+                             const float* const* sw2, void* C, int64_t ldc,
+                             const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg,
+                             int64_t N, int64_t K, int32_t epilogue,
+                             const void* R, int64_t ldr, const float* const* gate,
+                             const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
+                             void* stream);
 
 /* Tuning knob for measurements: selects a kernel variant by name ("attn", "gemm"); returns the
  * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default. */

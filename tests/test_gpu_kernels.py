@@ -162,6 +162,40 @@ def test_grouped_gemm_three_segments():
     assert_close(c, want, 0.99999, 6e-3, "grouped gemm")
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+def test_grouped_gemm_fp8_and_gaps(variant, request):
+    """e4m3 grouped launch: three segments with their own weights, one of them empty, rows outside every segment
+    untouched; the long segment spans several row tiles so the short ones share its grid."""
+    prev = ops.set_variant("gemm", variant)
+    request.addfinalizer(lambda: ops.set_variant("gemm", prev))
+    g = gen(123)
+    K, N, M = 512, 520, 900
+    segs = [(10, 600), (610, 0), (640, 200), (860, 40)]          # rows 0-9, 610-639, 840-859 belong to nobody
+    a, ar = rand_bf16((M, K), g)
+    aq, sa = ops.quant_rows(a)
+    ws = [rand_bf16((N, K), g, 0.05) for _ in segs]
+    qs = [ops.quant_rows(w[0]) for w in ws]
+    r, rr = rand_bf16((M, N), g)
+    gates = [torch.randn(N, generator=g), None, torch.randn(N, generator=g), None]
+    out = r.clone()
+    ops.grouped_gemm_fp8(aq, sa, [q[0] for q in qs], [q[1] for q in qs], segs, epilogue="gate_residual", residual=out,
+                         gates=[None if x is None else x.to(dev()) for x in gates], out=out)
+    want = rr.clone()
+    for i, (s0, ln) in enumerate(segs):
+        if ln:
+            want[s0:s0 + ln] = rr[s0:s0 + ln] + (1.0 if gates[i] is None else gates[i]) * O.fp8_linear(ar[s0:s0 + ln], ws[i][1])
+    assert_close(out, want, 0.99999, 6e-3, "grouped fp8 gemm")
+    for lo, hi in ((0, 10), (610, 640), (840, 860)):
+        assert torch.equal(out[lo:hi], r[lo:hi])
+    # the grouped launch equals the per-segment launches bit for bit
+    ref = r.clone()
+    for i, (s0, ln) in enumerate(segs):
+        if ln:
+            ops.gemm_fp8(aq[s0:s0 + ln], sa[s0:s0 + ln], qs[i][0], qs[i][1], epilogue="gate_residual", residual=ref[s0:s0 + ln],
+                         gate=None if gates[i] is None else gates[i].to(dev()), out=ref[s0:s0 + ln])
+    assert torch.equal(out, ref)
+
+
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("n,H,hd", [(64, 2, 64), (256, 1, 128), (1000, 3, 128), (321, 2, 64), (1, 1, 128), (130, 2, 128), (65, 1, 64),
