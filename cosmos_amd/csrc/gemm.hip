@@ -176,9 +176,33 @@ __device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) 
     return make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
 }
 
+constexpr int kStagePitch = 256 + 16;      // bytes per staged row (16-byte multiple; the pad spreads rows over banks)
+
+// wave-private staging area -> C: COLS (128 or 64) bf16 columns of 128 rows, whole rows per store instruction
+template <int COLS>
+__device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, const char* stage, int row0, int col0, int lane) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
+    constexpr int LPR = COLS / 8;                // lanes per row (16 bytes each)
+    constexpr int RPI = 64 / LPR;                // rows per instruction
+    const int rl = lane / LPR, ch = lane % LPR;
+    const int col = col0 + ch * 8;
+#pragma unroll
+    for (int it = 0; it < 128 / RPI; ++it) {
+        const int rloc = it * RPI + rl;
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + rloc * kStagePitch + ch * 16);
+        const int row = row0 + rloc;
+        if (row < t.m_end && col < p.N) *reinterpret_cast<uint4*>(p.C + (int64_t)row * p.ldc + col) = v;
+    }
+}
+
 template <int EPI, bool FP8>
 __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32x16 (&acc)[4][4], int m0, int n0, int wm,
-                                         int wn, int lane) {
+                                         int wn, int lane, char* stage) {
+    // `stage` (optional): kStagePitch * 128 bytes of LDS private to this wave.  The finished bf16 values then go
+    // there first and leave as whole rows, 16 bytes per lane: a store instruction covers 4 (SWIGLU: 8) output rows of
+    // 256 (128) contiguous bytes instead of 32 rows of 16 bytes.  All workgroups reach their epilogue at about the
+    // same time, so the epilogue runs at the HBM write rate; partial-line stores (which left the L2 as several
+    // writes per line when the row stride is a large power of two) made it up to four times longer.
     const int r32 = lane & 31, kh = lane >> 5;
     const int row_base = m0 + wm * 128 + r32;
     if (EPI == CDM_EPI_SWIGLU) {
@@ -206,9 +230,12 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         o[e] = silu_f(acc[mi][nj][4 * g + e] * sg[e]) * (acc[mi][nj + 2][4 * g + e] * su[e]);
-                    *reinterpret_cast<uint2*>(crow + col) = pack4_bf16(o[0], o[1], o[2], o[3]);
+                    const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
+                    if (stage) *reinterpret_cast<uint2*>(stage + (mi * 32 + r32) * kStagePitch + (nj * 32 + 8 * g + 4 * kh) * 2) = o2;
+                    else *reinterpret_cast<uint2*>(crow + col) = o2;
                 }
         }
+        if (stage) copy_out<64>(p, t, stage, m0 + wm * 128, n0 + wn * 64, lane);
         return;
     }
     const int col_base = n0 + wn * 128 + 4 * kh;
@@ -272,9 +299,12 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
                     o[2] = bf16lo(r2.y) + g4.z * o[2];
                     o[3] = bf16hi(r2.y) + g4.w * o[3];
                 }
-                *reinterpret_cast<uint2*>(crow + col) = pack4_bf16(o[0], o[1], o[2], o[3]);
+                const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
+                if (stage) *reinterpret_cast<uint2*>(stage + (mi * 32 + r32) * kStagePitch + (ni * 32 + 8 * g + 4 * kh) * 2) = o2;
+                else *reinterpret_cast<uint2*>(crow + col) = o2;
             }
     }
+    if (stage) copy_out<128>(p, t, stage, m0 + wm * 128, n0 + wn * 128, lane);
 }
 
 template <int EPI, bool FP8>
@@ -347,7 +377,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         compute_stage<FP8>(sa1, sb1, acc, wm, wn, lane);
     }
 
-    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane);
+    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -522,8 +552,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #undef CDM_RING_BARRIER
 #undef CDM_KSTEP
 #undef CDM_FENCE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // surplus loads must not outlive the workgroup's LDS
-    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane);
+    // surplus loads must not outlive the workgroup's LDS; after the barrier no wave reads the ring any more and
+    // each wave owns a quarter of it as the staging area of its epilogue
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane, s_ring + wave * (128 * kStagePitch));
 }
 
 // esize = bytes per operand element (2 = bf16, 1 = e4m3); strides in elements
