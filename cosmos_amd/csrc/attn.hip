@@ -444,25 +444,36 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         CDM_ATTN_STEP(s_b, s_a)
     }
 #undef CDM_ATTN_STEP
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct-to-LDS write may outlive the workgroup
-
+    // no direct-to-LDS write may outlive the workgroup; after the barrier no wave reads the K / V rings any more and
+    // each wave stages its output rows there, so that they leave as whole 2 * HD-byte rows (16 bytes per lane, 4 or 8 rows
+    // per store) instead of 8-byte pieces of 32 different rows
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    constexpr int PITCH = HD * 2 + 16;
+    static_assert((NW / 2) * 32 * QS * PITCH <= RING * TILE_BYTES, "staging area exceeds a ring");
+    char* stage = (wave < NW / 2 ? sk : sv) + (wave % (NW / 2)) * (32 * QS * PITCH);     // half the waves per ring
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
         const float l_tot = l_run[qs] + __shfl_xor(l_run[qs], 32, 64);
         const float inv = 1.0f / l_tot;
-        const int qrow = q0 + qs * 32 + r32;
-        if (qrow < p.n_tokens) {
-            bf16_t* op = p.o + (int64_t)qrow * p.ldo + head * HD + 4 * kh;
 #pragma unroll
-            for (int t = 0; t < HD / 32; ++t)
+        for (int t = 0; t < HD / 32; ++t)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    uint2 w;
-                    w.x = pack_bf16x2(oacc[qs][t][4 * g + 0] * inv, oacc[qs][t][4 * g + 1] * inv);
-                    w.y = pack_bf16x2(oacc[qs][t][4 * g + 2] * inv, oacc[qs][t][4 * g + 3] * inv);
-                    *reinterpret_cast<uint2*>(op + 32 * t + 8 * g) = w;
-                }
-        }
+            for (int g = 0; g < 4; ++g) {
+                uint2 w;
+                w.x = pack_bf16x2(oacc[qs][t][4 * g + 0] * inv, oacc[qs][t][4 * g + 1] * inv);
+                w.y = pack_bf16x2(oacc[qs][t][4 * g + 2] * inv, oacc[qs][t][4 * g + 3] * inv);
+                *reinterpret_cast<uint2*>(stage + (qs * 32 + r32) * PITCH + (32 * t + 8 * g + 4 * kh) * 2) = w;
+            }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
+    constexpr int LPR = HD / 8, RPI = 64 / LPR;             // lanes per row, rows per store instruction
+    const int rl = lane / LPR, ch = lane % LPR;
+#pragma unroll
+    for (int it = 0; it < 32 * QS / RPI; ++it) {
+        const int rloc = it * RPI + rl;
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + rloc * PITCH + ch * 16);
+        const int qrow = q0 + rloc;
+        if (qrow < p.n_tokens) *reinterpret_cast<uint4*>(p.o + (int64_t)qrow * p.ldo + head * HD + ch * 8) = v;
     }
 }
 
@@ -647,7 +658,7 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     if ((rc = make_qk_norm("attn_fwd_packed", qk_norm, 0, n_tokens, &qn))) return rc;
     const int64_t d = (int64_t)n_heads * head_dim;
     CDM_REQUIRE(ldq >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd_packed: row stride smaller than n_heads*head_dim");
-    CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(workspace) && cdm_aligned16(o) && ldq % 8 == 0 && ldo % 4 == 0,
+    CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(workspace) && cdm_aligned16(o) && ldq % 8 == 0 && ldo % 8 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd_packed: pointers/strides must be 16-byte aligned");
     if (n_tokens == 0) return CDM_OK;
     if ((rc = cdm_require_device())) return rc;
@@ -699,7 +710,7 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
     CDM_REQUIRE(causal_prefix >= 0 && causal_prefix <= n_tokens, CDM_ERR_BAD_ARG,
                 "attn_fwd: causal_prefix=%lld outside [0, n_tokens]", (long long)causal_prefix);
     CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(o) && ldq % 8 == 0 &&
-                    ldk % 8 == 0 && ldv % 8 == 0 && ldo % 4 == 0,
+                    ldk % 8 == 0 && ldv % 8 == 0 && ldo % 8 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
     if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_heads, head_dim,
                                     qk_norm, stream)))
