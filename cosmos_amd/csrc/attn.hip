@@ -489,7 +489,9 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
     constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
     constexpr int HALF = HD / 2;
     constexpr int TILE_BYTES = BN * HD * 2;
-    const int tile_idx = blockIdx.x, head = blockIdx.y;
+    // heads vary fastest over the grid: the K / V rows of neighbouring heads are adjacent in memory, so the
+    // workgroups that run together share DRAM pages and cache lines
+    const int tile_idx = blockIdx.y, head = blockIdx.x;
     const int t0 = tile_idx * 64;
     char* kt = kp + ((int64_t)head * n_tiles + tile_idx) * TILE_BYTES;
     char* vt = vp + ((int64_t)head * n_tiles + tile_idx) * TILE_BYTES;
@@ -592,7 +594,7 @@ int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, in
                           const float* sin) {
     CDM_REQUIRE(n_tokens >= 0 && n_heads > 0, CDM_ERR_BAD_ARG, "%s: bad sizes", who);
     CDM_REQUIRE(head_dim == 64 || head_dim == 128, CDM_ERR_BAD_SHAPE, "%s: head_dim=%d must be 64 or 128", who, head_dim);
-    CDM_REQUIRE(n_tokens < (1ll << 23) && n_heads <= 65535, CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
+    CDM_REQUIRE(n_tokens <= 65535ll * BN && n_heads <= 65535, CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
     CDM_REQUIRE((cos == nullptr) == (sin == nullptr), CDM_ERR_BAD_ARG, "%s: cos and sin must be given together", who);
     CDM_REQUIRE(cdm_aligned16(cos) && cdm_aligned16(sin), CDM_ERR_BAD_ALIGN, "%s: rotary tables must be 16-byte aligned", who);
     return CDM_OK;
@@ -627,7 +629,7 @@ extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void*
     const int n_tiles = (int)(pad_tokens(n_tokens) / BN);
     const int64_t img = image_bytes(n_tokens, n_heads, head_dim);
     char* ws = (char*)workspace;
-    dim3 grid(n_tiles, n_heads);
+    dim3 grid(n_heads, n_tiles);
     hipStream_t st = (hipStream_t)stream;
     if (head_dim == 128)
         pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, kn, ws, ws + img,
