@@ -423,18 +423,23 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     {                                                                                                           \
         const int k_fill = vs_cur;                              /* slot of K(j)   == j % 3     */               \
         const int v_fill = ks_next == 2 ? 0 : ks_next + 1;      /* slot of V(j-1) == (j+2) % 3 */               \
-        auto sync = [&]() {                                                                                     \
+        /* the K loads go out at the synchronisation point, the V loads half a step later: two bursts of two   */ \
+        /* loads per wave instead of one of four (a wave sits in the vector-memory issue queue while its loads   */ \
+        /* are accepted); both tiles were released by the same barrier                                           */ \
+        auto sync_k = [&]() {                                                                                   \
             asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory");                       \
             issue(kbase, kpre, sk_addr, j + 3, k_fill);                                                         \
-            issue(vbase, vpre, sv_addr, j + 2, v_fill);                                                         \
         };                                                                                                      \
-        if (!late_sync) sync();                                                                                 \
+        auto load_v = [&]() { issue(vbase, vpre, sv_addr, j + 2, v_fill); };                                    \
+        if (!late_sync) sync_k();                                                                               \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QS];                                                                                         \
         _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS>([&]() { if (late_sync) sync(); }, sk + ks_next * TILE_BYTES, sv + vs_cur * TILE_BYTES, \
-                          sk + v_fill * TILE_BYTES, qf, kw,                                                     \
+        pipe_step<HD, QS>([&]() { if (late_sync) sync_k(); else load_v(); }, sk + ks_next * TILE_BYTES,         \
+                          sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,                           \
                           SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 == NT), nvalid);  \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        if (late_sync) load_v();                                                                                \
         vs_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
