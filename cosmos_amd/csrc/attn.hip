@@ -102,13 +102,14 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 // the top of the step releases the wave, and all softmax arithmetic is placed under MFMAs:
 //   block A  : S(j+1) = K(j+1) Q^T - m_ref, 16 MFMAs seeded with -m_ref (rolling K fragment window, first
 //              KWIN k-steps preloaded in the previous step)
-//              ||  p = exp2(s_cur), bf16 pack, row sum of tile j ; first V^T fragments of tile j
+//              ||  p = exp2(s_cur), bf16 pack, row sum of tile j
+//   middle   : (barrier of the out-of-phase waves) ; first V^T fragments of tile j ; tile loads
 //   block B  : O^T += V^T P^T, 16 MFMAs (rolling V^T window)
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-template <int HD, int QS, class Mid>
-__device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
+template <int HD, int QS, class Pre, class Post>
+__device__ __forceinline__ void pipe_step(Pre&& mid_pre, Post&& mid_post, const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
                                           f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
@@ -151,9 +152,6 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
         }
         l_run[qs] += psum;
     }
-    bf16x8 vw[VWIN];
-#pragma unroll
-    for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
     // per MFMA (at most) one fragment read and six VALU instructions
 #pragma unroll
     for (int i = 0; i < 2 * KS * QS; ++i) {
@@ -167,7 +165,13 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
     for (int qs = 0; qs < QS; ++qs)
         asm volatile("" : "+v"(pf[qs][0]), "+v"(pf[qs][1]), "+v"(pf[qs][2]), "+v"(pf[qs][3]), "+v"(l_run[qs]));
     __builtin_amdgcn_sched_barrier(0);
-    mid();                 // the step's synchronisation point for the waves that take it between the two blocks
+    mid_pre();             // the step's synchronisation point for the waves that take it between the two blocks
+    // V(j) is only known to have landed after the step's barrier, so its first fragments are read behind the
+    // synchronisation point of either kind of wave; the tile loads issued next cover the LDS latency
+    bf16x8 vw[VWIN];
+#pragma unroll
+    for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
+    mid_post();
     __builtin_amdgcn_sched_barrier(0);
     if (next_masked) {     // wave-uniform: before a ragged last tile, and in every step of a causal query block
 #pragma unroll
@@ -243,7 +247,7 @@ struct PackedParams {
     bf16_t* o; int64_t ldo;
     const float* cos; const float* sin;   // optional rotary tables [n_tokens, HD/2] applied to Q at load
     QkNormDev qn;                          // optional per-head RMSNorm of Q, applied before the rotation
-    int n_tokens, n_heads;
+    int n_tokens, n_heads, n_qblocks;
     float scale_log2e;
 };
 
@@ -263,8 +267,19 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r32 = lane & 31, kh = lane >> 5;
-    const int head = blockIdx.y;
-    const int q0 = blockIdx.x * BMQ + wave * (32 * QS);
+    // XCD-aware placement: workgroup ids are dealt round-robin over the 8 XCDs.  All query blocks of a head go to
+    // ONE XCD (head % 8), so a head's K / V tile images are fetched into one L2 instead of eight.
+    int head, qblk;
+    {
+        const int nqb = p.n_qblocks, nh = p.n_heads;
+        const int xcd = blockIdx.x & 7, k = blockIdx.x >> 3;      // k-th workgroup of its XCD
+        const int hpx = (nh + 7) >> 3;                            // heads per XCD (last XCDs may own one less)
+        const int hi = k / nqb;
+        head = hi * 8 + xcd;
+        qblk = k - hi * nqb;
+        if (hi >= hpx || head >= nh) return;
+    }
+    const int q0 = qblk * BMQ + wave * (32 * QS);
 
     // ---- Q fragments: rotate-half mRoPE (if tables are given) and the factor log2(e)/sqrt(HD), both in fp32 and
     // with ONE rounding to bf16.  The lane holds channels 16ks + 8kh .. +7 of its query row for every ks, so
@@ -353,7 +368,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     const int last_valid = n_keys - (NT - 1) * BN;
     // per-row key limit and the tiles this workgroup needs: a query block inside the causal prefix stops at its
     // own last row, and every tile it visits is masked per row
-    const int b0 = blockIdx.x * BMQ;
+    const int b0 = qblk * BMQ;
     const bool causal_wg = b0 < p.causal_prefix;
     int klim[QS];
 #pragma unroll
@@ -426,16 +441,15 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         /* the K loads go out at the synchronisation point, the V loads half a step later: two bursts of two   */ \
         /* loads per wave instead of one of four (a wave sits in the vector-memory issue queue while its loads   */ \
         /* are accepted); both tiles were released by the same barrier                                           */ \
-        auto sync_k = [&]() {                                                                                   \
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory");                       \
-            issue(kbase, kpre, sk_addr, j + 3, k_fill);                                                         \
-        };                                                                                                      \
+        auto sync = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory"); };      \
+        auto load_k = [&]() { issue(kbase, kpre, sk_addr, j + 3, k_fill); };                                    \
         auto load_v = [&]() { issue(vbase, vpre, sv_addr, j + 2, v_fill); };                                    \
-        if (!late_sync) sync_k();                                                                               \
+        if (!late_sync) { sync(); load_k(); }                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QS];                                                                                         \
         _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS>([&]() { if (late_sync) sync_k(); else load_v(); }, sk + ks_next * TILE_BYTES,         \
+        pipe_step<HD, QS>([&]() { if (late_sync) sync(); }, [&]() { if (late_sync) load_k(); else load_v(); },  \
+                          sk + ks_next * TILE_BYTES,                                                            \
                           sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,                           \
                           SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 == NT), nvalid);  \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
@@ -682,7 +696,11 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     p.qn = qn;
     p.n_tokens = (int)n_tokens; p.n_heads = n_heads;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
-    dim3 grid((unsigned)((n_tokens + BMQ - 1) / BMQ), n_heads);
+    p.n_qblocks = (int)((n_tokens + BMQ - 1) / BMQ);
+    // 1-D grid of 8 x ceil(heads / 8) x query blocks ids: id % 8 = XCD, see the kernel's placement rule
+    const int64_t nwg = 8ll * ((n_heads + 7) / 8) * p.n_qblocks;
+    CDM_REQUIRE(nwg < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd_packed: grid too large");
+    dim3 grid((unsigned)nwg);
     hipStream_t st = (hipStream_t)stream;
     // variant 0 = 32 query rows per wave (8 waves, two per SIMD); 1 = 64 query rows per wave (4 waves)
     if (cdm_get_variant(0) == 1) {
