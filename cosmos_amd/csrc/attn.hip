@@ -102,14 +102,15 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 // the top of the step releases the wave, and all softmax arithmetic is placed under MFMAs:
 //   block A  : S(j+1) = K(j+1) Q^T - m_ref, 16 MFMAs seeded with -m_ref (rolling K fragment window, first
 //              KWIN k-steps preloaded in the previous step)
-//              ||  p = exp2(s_cur), bf16 pack, row sum of tile j
-//   middle   : (barrier of the out-of-phase waves) ; first V^T fragments of tile j ; tile loads
+//              ||  p = exp2(s_cur), bf16 pack, row sum of tile j ; first V^T fragments of tile j (a wave that
+//              takes the step's barrier behind block A reads them before that barrier: V(j) is complete one
+//              barrier early)
 //   block B  : O^T += V^T P^T, 16 MFMAs (rolling V^T window)
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-template <int HD, int QS, class Pre, class Post>
-__device__ __forceinline__ void pipe_step(Pre&& mid_pre, Post&& mid_post, const char* sk_next, const char* sv_cur, const char* sk_next2,
+template <int HD, int QS, class Mid>
+__device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
                                           f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
@@ -152,6 +153,9 @@ __device__ __forceinline__ void pipe_step(Pre&& mid_pre, Post&& mid_post, const 
         }
         l_run[qs] += psum;
     }
+    bf16x8 vw[VWIN];
+#pragma unroll
+    for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
     // per MFMA (at most) one fragment read and six VALU instructions
 #pragma unroll
     for (int i = 0; i < 2 * KS * QS; ++i) {
@@ -165,13 +169,7 @@ __device__ __forceinline__ void pipe_step(Pre&& mid_pre, Post&& mid_post, const 
     for (int qs = 0; qs < QS; ++qs)
         asm volatile("" : "+v"(pf[qs][0]), "+v"(pf[qs][1]), "+v"(pf[qs][2]), "+v"(pf[qs][3]), "+v"(l_run[qs]));
     __builtin_amdgcn_sched_barrier(0);
-    mid_pre();             // the step's synchronisation point for the waves that take it between the two blocks
-    // V(j) is only known to have landed after the step's barrier, so its first fragments are read behind the
-    // synchronisation point of either kind of wave; the tile loads issued next cover the LDS latency
-    bf16x8 vw[VWIN];
-#pragma unroll
-    for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
-    mid_post();
+    mid();                 // the step's synchronisation point for the waves that take it between the two blocks
     __builtin_amdgcn_sched_barrier(0);
     if (next_masked) {     // wave-uniform: before a ragged last tile, and in every step of a causal query block
 #pragma unroll
@@ -260,9 +258,12 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     constexpr int NW = 8 / QS;
     constexpr int TILE_BYTES = BN * HD * 2;            // same for K and V tiles
     constexpr int PER_WAVE = TILE_BYTES / 1024 / NW;   // direct-to-LDS instructions per wave per tile
-    constexpr int RING = 3;                            // K(t) lives in slot t % 3, V(t) in slot t % 3
+    // K(t) lives in slot t % 3 and V(t) in slot t % 4.  V is loaded one step further ahead than its first use by
+    // the in-phase waves needs: the out-of-phase waves read the first fragments of V(j) BEFORE barrier j, so V(j)
+    // has to be complete at barrier j - 1
+    constexpr int RING = 3, RING_V = 4;
     __shared__ __attribute__((aligned(1024))) char sk[RING * TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char sv[RING * TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char sv[RING_V * TILE_BYTES];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -395,13 +396,14 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             lds_dma16(src + i * (NW * 1024), lane_off, dst_addr + slot * TILE_BYTES + i * (NW * 1024));
     };
 
-    // ---- prologue: K(0) | K(1), V(0) | K(2), V(1); scores of tile 0 with an exact first reference
+    // ---- prologue: K(0) | K(1), V(0) | K(2), V(1) | V(2); scores of tile 0 with an exact first reference
     issue(kbase, kpre, sk_addr, 0, 0);
     issue(kbase, kpre, sk_addr, 1, 1);
     issue(vbase, vpre, sv_addr, 0, 0);
     issue(kbase, kpre, sk_addr, 2, 2);
     issue(vbase, vpre, sv_addr, 1, 1);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
+    issue(vbase, vpre, sv_addr, 2, 2);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(3 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
     f32x16 s_a[QS][2], s_b[QS][2];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
 #pragma unroll
@@ -421,40 +423,41 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     bf16x8 kw[KWIN][2];
     preload_k<HD>(sk + TILE_BYTES, kw, lane);      // K(1) for step 0
 
-    // step j: S(j+1) from K slot (j+1)%3, P(j) V(j) from V slot j%3, K(j+2) fragments preloaded from slot (j+2)%3.
-    // At the barrier everything but the most recently issued group, V(j+1), must have landed
-    // (s_waitcnt vmcnt(1 tile)): K(j+2) is read at the end of this very step.  After the barrier every wave is
-    // done with K(j) and V(j-1), whose slots are refilled with K(j+3) and V(j+2).
-    int ks_next = 1, vs_cur = 0;      // ring slots: (j+1)%3 and j%3
+    // step j: S(j+1) from K slot (j+1)%3, P(j) V(j) from V slot j%4, K(j+2) fragments preloaded from slot (j+2)%3.
+    // At the barrier everything but the most recently issued group, V(j+2), must have landed
+    // (s_waitcnt vmcnt(1 tile)): K(j+2) is read at the end of this very step and the first fragments of V(j+1)
+    // possibly before the next barrier.  After the barrier every wave is done with K(j) and V(j-1), whose slots
+    // are refilled with K(j+3) and V(j+3).
+    int ks_next = 1, ks_cur = 0;      // K ring slots (j+1)%3 and j%3
     // Two waves share a SIMD (wave w and w + 4).  Block A of a step is VALU-heavy (exp, pack) and block B is pure
     // MFMA; if both waves of a SIMD took the step's barrier at the same point they would need the VALU together and
     // the matrix pipe together.  So the upper four waves take the SAME barrier between block A and block B
     // instead of in front of block A: they run half a step out of phase, and while one wave of a SIMD is in its
-    // VALU-heavy block the other is in its MFMA block.  Tile lifetimes do not change: a wave still reads K(j+1) and
-    // K(j+2) fragments and V(j) between the barriers that bracket those tiles (K(j+1) has landed one barrier
-    // earlier than the in-phase waves need it).
+    // VALU-heavy block the other is in its MFMA block.  Such a wave reads K(j+1) and the first fragments of V(j)
+    // before barrier j: both tiles are complete at barrier j - 1 (neither is the most recently issued group there),
+    // and their slots are not refilled before barrier j + 1.
     const bool late_sync = QS == 1 && wave >= 4;
 #define CDM_ATTN_STEP(SCUR, SNEXT)                                                                              \
     {                                                                                                           \
-        const int k_fill = vs_cur;                              /* slot of K(j)   == j % 3     */               \
-        const int v_fill = ks_next == 2 ? 0 : ks_next + 1;      /* slot of V(j-1) == (j+2) % 3 */               \
+        const int k_fill = ks_cur;                              /* slot of K(j)   == j % 3     */               \
+        const int k_next2 = ks_next == 2 ? 0 : ks_next + 1;     /* slot of K(j+2) == (j+2) % 3 */               \
+        const int v_cur = j & 3, v_fill = (j + 3) & 3;          /* slots of V(j) and of V(j-1) */               \
         /* the K loads go out at the synchronisation point, the V loads half a step later: two bursts of two   */ \
         /* loads per wave instead of one of four (a wave sits in the vector-memory issue queue while its loads   */ \
         /* are accepted); both tiles were released by the same barrier                                           */ \
         auto sync = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER_WAVE) : "memory"); };      \
         auto load_k = [&]() { issue(kbase, kpre, sk_addr, j + 3, k_fill); };                                    \
-        auto load_v = [&]() { issue(vbase, vpre, sv_addr, j + 2, v_fill); };                                    \
+        auto load_v = [&]() { issue(vbase, vpre, sv_addr, j + 3, v_fill); };                                    \
         if (!late_sync) { sync(); load_k(); }                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QS];                                                                                         \
         _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS>([&]() { if (late_sync) sync(); }, [&]() { if (late_sync) load_k(); else load_v(); },  \
-                          sk + ks_next * TILE_BYTES,                                                            \
-                          sv + vs_cur * TILE_BYTES, sk + v_fill * TILE_BYTES, qf, kw,                           \
+        pipe_step<HD, QS>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },                       \
+                          sk + ks_next * TILE_BYTES, sv + v_cur * TILE_BYTES, sk + k_next2 * TILE_BYTES, qf, kw, \
                           SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 == NT), nvalid);  \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         if (late_sync) load_v();                                                                                \
-        vs_cur = ks_next;                                                                                       \
+        ks_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
     for (int j = 0; j < NTW; ++j) {

@@ -235,6 +235,12 @@ def test_c1_full_size_attention_sampled_rows():
     vmin, vmax = v.float().amin(0), v.float().amax(0)
     of = o.float()
     assert bool((of >= vmin - 1e-2).all()) and bool((of <= vmax + 1e-2).all())
+    # the kernel has no atomics and a fixed summation order: repeated launches agree bit for bit.  A tile read
+    # before it has landed in LDS shows up here as a last-bit difference in a few rows (one tile of 880 is
+    # below the bf16 resolution of the output, so the comparison with the oracle above cannot see it).
+    for _ in range(4):
+        again = ops.attention(q, k, v, H, hd, cos=cos.to(dev()), sin=sin.to(dev()))
+        assert torch.equal(o, again), "attention output differs between identical launches"
 
 
 def test_transformer_with_stack_edges_and_loaded_checkpoint(tmp_path):
