@@ -384,3 +384,32 @@ def test_c2_full_size_gemms_sampled_rows(fp8):
     if not fp8:
         # linearity at full size: gemm(2x) == 2 gemm(x) exactly (a power of two commutes with every rounding)
         assert torch.equal(ops.gemm(x * 2, wo), qkv.new_tensor(2.0) * ops.gemm(x, wo))
+
+
+@pytest.mark.parametrize("name", ["C2", "C3", "C4"])
+def test_full_size_block_is_bit_reproducible(name):
+    """One block of each full-size benchmark configuration, run four times on the same input.  No kernel on the path
+    uses atomics or an order that depends on timing, so the outputs must agree bit for bit; a difference means
+    that some wave read a tile (LDS ring slot, staged row) before it was complete."""
+    import dataclasses
+    cfg = dataclasses.replace(CONFIGS[name], n_blocks=1)
+    st = DMStack(cfg, device=dev())
+    st.reset_parameters()
+    g = torch.Generator(device=dev()).manual_seed(7)
+    with torch.no_grad():
+        for b in st.blocks:
+            b.adaLN_modulation.bias.copy_(0.5 * torch.randn(b.adaLN_modulation.bias.shape, generator=g, device=dev()))
+    mk = lambda n: torch.randn((1, n, cfg.d_model), generator=g, device=dev()).to(torch.bfloat16)
+    x, kw = mk(cfg.n_video), {}
+    if cfg.n_text:
+        kw["encoder_hidden_states"] = mk(cfg.n_text)
+    if cfg.n_action:
+        kw["action_states"] = mk(cfg.n_action)
+    t = torch.tensor([500.0], device=dev())
+    (first,) = st(x, t, **kw)
+    first = first.clone()
+    assert bool(torch.isfinite(first.float()).all())
+    assert float((first.float() - x.float()).abs().max()) > 0.1          # the block does something
+    for _ in range(3):
+        (again,) = st(x, t, **kw)
+        assert torch.equal(first, again), f"{name}: block output differs between identical launches"
