@@ -69,7 +69,7 @@ def test_mrope_standalone(hd, H, sections):
 # ------------------------------------------------------------------ GEMM
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (8, 8, 128), (300, 264, 256), (1024, 3072, 1024), (515, 1000, 384),
-                                   (257, 520, 4096)])
+                                   (257, 520, 4096), (4100, 4360, 256)])      # the last: 306 tiles, more than the chip has CUs
 def test_gemm_plain(M, N, K, variant):
     g = gen(M + N + K)
     a, ar = rand_bf16((M, K), g)
@@ -96,7 +96,7 @@ def test_gemm_strided_views_and_determinism():
 
 
 @pytest.mark.parametrize("variant", [0, 1])
-@pytest.mark.parametrize("M,N,K", [(256, 128, 128), (333, 200, 256), (1024, 4096, 1024)])
+@pytest.mark.parametrize("M,N,K", [(256, 128, 128), (333, 200, 256), (1024, 4096, 1024), (4100, 2184, 256)])
 def test_gemm_swiglu(M, N, K, variant, request):
     prev = ops.set_variant("gemm", variant)
     request.addfinalizer(lambda: ops.set_variant("gemm", prev))
@@ -110,7 +110,8 @@ def test_gemm_swiglu(M, N, K, variant, request):
 
 
 @pytest.mark.parametrize("variant", [0, 1])
-@pytest.mark.parametrize("M,N,K,gated", [(256, 256, 128, True), (300, 1024, 512, True), (77, 264, 128, False)])
+@pytest.mark.parametrize("M,N,K,gated", [(256, 256, 128, True), (300, 1024, 512, True), (77, 264, 128, False),
+                                         (4100, 4360, 128, True)])
 def test_gemm_gate_residual(M, N, K, gated, variant, request):
     prev = ops.set_variant("gemm", variant)
     request.addfinalizer(lambda: ops.set_variant("gemm", prev))
@@ -358,7 +359,8 @@ def test_adaln_rmsnorm_quant():
 
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("M,N,K,epi", [(256, 256, 256, "none"), (300, 520, 512, "none"), (300, 264, 256, "swiglu"),
-                                       (130, 256, 256, "gate_residual"), (515, 1000, 1792, "none")])
+                                       (130, 256, 256, "gate_residual"), (515, 1000, 1792, "none"),
+                                       (4100, 4360, 256, "none"), (4100, 2184, 256, "swiglu")])
 def test_gemm_fp8(M, N, K, epi, variant, request):
     prev = ops.set_variant("gemm", variant)
     request.addfinalizer(lambda: ops.set_variant("gemm", prev))
