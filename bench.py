@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0
 # rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a plain streaming
 # kernel of known size (FETCH_SIZE unit = 2 KiB, WRITE_SIZE unit = 1 KiB on this chip).  Counters cannot be read
 # from inside this process, so other shapes report null.
-ATTN_TRAFFIC_BYTES = {(56832, 32, 128): 14.84e9 + 0.466e9}
+ATTN_TRAFFIC_BYTES = {(56832, 32, 128): 8.61e9 + 0.466e9}
 
 
 def cpu_baseline(cfg, sample_tokens: int):
