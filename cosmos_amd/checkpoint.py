@@ -107,7 +107,10 @@ def load_generator_weights(model, source: Union[str, Iterable[str], Mapping[str,
                     continue
                 blk = stack.blocks[layer]
                 if tgt[0] == "qkv":
-                    blk.attn.qkv_weight[br].data[tgt[1] * d:(tgt[1] + 1) * d].copy_(t)
+                    # rows of the fused weight: [q: d | k: d_kv | v: d_kv] (d_kv < d under grouped-query attention)
+                    dkv = blk.attn.n_kv_heads * blk.attn.head_dim
+                    r0 = (0, d, d + dkv)[tgt[1]]
+                    blk.attn.qkv_weight[br].data[r0:r0 + (d if tgt[1] == 0 else dkv)].copy_(t)
                     seen.add(f"layers.{layer}.qkv.{br}.{tgt[1]}")
                 elif tgt[0] == "attn":
                     getattr(blk.attn, tgt[1])[br].data.copy_(t)
@@ -172,8 +175,9 @@ def export_generator_weights(model) -> Dict[str, torch.Tensor]:
         for b in range(min(stack.cfg.n_branches, 2)):
             q, k, v, o, nq, nk = names[b]
             w = blk.attn.qkv_weight[b].data
-            out[pre + f"self_attn.{q}.weight"], out[pre + f"self_attn.{k}.weight"] = w[:d].clone(), w[d:2 * d].clone()
-            out[pre + f"self_attn.{v}.weight"] = w[2 * d:].clone()
+            dkv = blk.attn.n_kv_heads * blk.attn.head_dim
+            out[pre + f"self_attn.{q}.weight"], out[pre + f"self_attn.{k}.weight"] = w[:d].clone(), w[d:d + dkv].clone()
+            out[pre + f"self_attn.{v}.weight"] = w[d + dkv:].clone()
             out[pre + f"self_attn.{o}.weight"] = blk.attn.out_weight[b].data.clone()
             if blk.attn.qk_norm:
                 out[pre + f"self_attn.{nq}.weight"] = blk.attn.norm_q_weight.data[b].clone()

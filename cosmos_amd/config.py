@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Tuple
+from typing import Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -24,7 +24,12 @@ class DMConfig:
     fp8: bool = False
     qk_norm: bool = False                    # per-head RMSNorm of Q and K ahead of the rotation
     hybrid_mask: bool = False                # text run causal and blind to the generator tokens (else full attention)
+    n_kv_heads: Optional[int] = None         # K / V heads (None = n_heads; fewer = grouped-query attention)
     seed: int = 1234
+
+    @property
+    def kv_heads(self) -> int:
+        return self.n_heads if self.n_kv_heads is None else self.n_kv_heads
 
     @property
     def n_video(self) -> int:

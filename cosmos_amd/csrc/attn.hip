@@ -236,7 +236,7 @@ struct QkNormDev {
 
 struct PackedParams {
     const bf16_t* q; int64_t ldq;
-    const char* kp;              // [n_heads][n_tiles][tile bytes]
+    const char* kp;              // [n_kv_heads][n_tiles][tile bytes]
     const char* vp;
     const char* kp_prefix;       // optional tile images of keys that precede those of kp / vp (whole tiles)
     const char* vp_prefix;
@@ -246,6 +246,7 @@ struct PackedParams {
     const float* cos; const float* sin;   // optional rotary tables [n_tokens, HD/2] applied to Q at load
     QkNormDev qn;                          // optional per-head RMSNorm of Q, applied before the rotation
     int n_tokens, n_heads, n_qblocks;
+    int kv_group;                // query heads per K / V head (1 = multi-head attention)
     float scale_log2e;
 };
 
@@ -269,17 +270,19 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r32 = lane & 31, kh = lane >> 5;
     // XCD-aware placement: workgroup ids are dealt round-robin over the 8 XCDs.  All query blocks of a head go to
-    // ONE XCD (head % 8), so a head's K / V tile images are fetched into one L2 instead of eight.
+    // ONE XCD, so a head's K / V tile images are fetched into one L2 instead of eight, and an XCD owns a contiguous
+    // range of heads, so the query heads that share a K / V head (grouped-query attention) share an L2 as well.
     int head, qblk;
     {
         const int nqb = p.n_qblocks, nh = p.n_heads;
         const int xcd = blockIdx.x & 7, k = blockIdx.x >> 3;      // k-th workgroup of its XCD
-        const int hpx = (nh + 7) >> 3;                            // heads per XCD (last XCDs may own one less)
+        const int hpx = (nh + 7) >> 3;                            // heads per XCD (the last XCDs may own fewer)
         const int hi = k / nqb;
-        head = hi * 8 + xcd;
+        head = xcd * hpx + hi;
         qblk = k - hi * nqb;
         if (hi >= hpx || head >= nh) return;
     }
+    const int kv_head = head / p.kv_group;
     const int q0 = qblk * BMQ + wave * (32 * QS);
 
     // ---- Q fragments: rotate-half mRoPE (if tables are given) and the factor log2(e)/sqrt(HD), both in fp32 and
@@ -380,10 +383,10 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     const int kmax = (causal_wg && b0 + BMQ <= p.causal_prefix) ? (b0 + BMQ < n_keys ? b0 + BMQ : n_keys) : n_keys;
     const int NTW = (kmax + BN - 1) / BN;
     const uint32_t lane_off = (uint32_t)(wave * 1024 + lane * 16);
-    const char* kbase = p.kp + (int64_t)head * NM * TILE_BYTES;
-    const char* vbase = p.vp + (int64_t)head * NM * TILE_BYTES;
-    const char* kpre = p.kp_prefix + (int64_t)head * NP * TILE_BYTES;
-    const char* vpre = p.vp_prefix + (int64_t)head * NP * TILE_BYTES;
+    const char* kbase = p.kp + (int64_t)kv_head * NM * TILE_BYTES;
+    const char* vbase = p.vp + (int64_t)kv_head * NM * TILE_BYTES;
+    const char* kpre = p.kp_prefix + (int64_t)kv_head * NP * TILE_BYTES;
+    const char* vpre = p.vp_prefix + (int64_t)kv_head * NP * TILE_BYTES;
     const uint32_t sk_addr = lds_addr_of(sk) + wave * 1024, sv_addr = lds_addr_of(sv) + wave * 1024;
 
     // tile `t` (clamped to the last tile, so that every step issues the same number of loads and the
@@ -624,7 +627,7 @@ int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, in
 
 }  // namespace
 
-// workspace = [Kp | Vp]: the two tile images
+// workspace = [Kp | Vp]: the two tile images; n_heads counts K / V heads
 extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
     if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0) return 0;
     return 2 * image_bytes(n_tokens, n_heads, head_dim);
@@ -664,10 +667,12 @@ extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void*
 
 extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
                                             const void* workspace, void* o, int64_t ldo, int64_t n_tokens,
-                                            int32_t n_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
-                                            const void* prefix_workspace, int64_t n_prefix_tokens,
-                                            int64_t causal_prefix, void* stream) {
+                                            int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
+                                            const cdm_qk_norm* qk_norm, const void* prefix_workspace,
+                                            int64_t n_prefix_tokens, int64_t causal_prefix, void* stream) {
     CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
+    CDM_REQUIRE(n_kv_heads > 0 && n_heads > 0 && n_heads % n_kv_heads == 0, CDM_ERR_BAD_SHAPE,
+                "attn_fwd_packed: n_kv_heads=%d must divide n_heads=%d", n_kv_heads, n_heads);
     CDM_REQUIRE(n_prefix_tokens >= 0 && n_prefix_tokens % BN == 0 && n_prefix_tokens < (1ll << 23), CDM_ERR_BAD_SHAPE,
                 "attn_fwd_packed: n_prefix_tokens=%lld must be a non-negative multiple of %d", (long long)n_prefix_tokens, BN);
     CDM_REQUIRE((n_prefix_tokens > 0) == (prefix_workspace != nullptr) && cdm_aligned16(prefix_workspace), CDM_ERR_BAD_ARG,
@@ -686,18 +691,18 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
                 CDM_ERR_BAD_ALIGN, "attn_fwd_packed: pointers/strides must be 16-byte aligned");
     if (n_tokens == 0) return CDM_OK;
     if ((rc = cdm_require_device())) return rc;
-    const int64_t img = image_bytes(n_tokens, n_heads, head_dim);
+    const int64_t img = image_bytes(n_tokens, n_kv_heads, head_dim);
     PackedParams p;
     p.q = (const bf16_t*)q; p.ldq = ldq;
     p.kp = (const char*)workspace; p.vp = (const char*)workspace + img;
     p.kp_prefix = (const char*)prefix_workspace;
-    p.vp_prefix = (const char*)prefix_workspace + image_bytes(n_prefix_tokens, n_heads, head_dim);
+    p.vp_prefix = (const char*)prefix_workspace + image_bytes(n_prefix_tokens, n_kv_heads, head_dim);
     p.n_prefix_tiles = (int)(n_prefix_tokens / BN);
     p.causal_prefix = (int)causal_prefix;
     p.o = (bf16_t*)o; p.ldo = ldo;
     p.cos = cos; p.sin = sin;
     p.qn = qn;
-    p.n_tokens = (int)n_tokens; p.n_heads = n_heads;
+    p.n_tokens = (int)n_tokens; p.n_heads = n_heads; p.kv_group = n_heads / n_kv_heads;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
     p.n_qblocks = (int)((n_tokens + BMQ - 1) / BMQ);
     // 1-D grid of 8 x ceil(heads / 8) x query blocks ids: id % 8 = XCD, see the kernel's placement rule
@@ -718,31 +723,34 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
 
 extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                                      int64_t ldv, const float* cos, const float* sin, void* o, int64_t ldo,
-                                     int64_t n_tokens, int32_t n_heads, int32_t head_dim, void* workspace,
-                                     int64_t workspace_bytes, const cdm_qk_norm* qk_norm, int64_t causal_prefix,
-                                     void* stream) {
+                                     int64_t n_tokens, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
+                                     void* workspace, int64_t workspace_bytes, const cdm_qk_norm* qk_norm,
+                                     int64_t causal_prefix, void* stream) {
     CDM_REQUIRE(q && k && v && o, CDM_ERR_BAD_ARG, "attn_fwd: null pointer");
     int32_t rc = check_attn_common("attn_fwd", n_tokens, n_heads, head_dim, cos, sin);
     if (rc) return rc;
+    CDM_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, CDM_ERR_BAD_SHAPE,
+                "attn_fwd: n_kv_heads=%d must divide n_heads=%d", n_kv_heads, n_heads);
     {
         QkNormDev tmp;
         if ((rc = make_qk_norm("attn_fwd", qk_norm, 0, n_tokens, &tmp))) return rc;
     }
     if (n_tokens == 0) return CDM_OK;
-    const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim);
+    const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim);
     CDM_REQUIRE(workspace && cdm_aligned16(workspace) && workspace_bytes >= need, CDM_ERR_BAD_ARG,
                 "attn_fwd: workspace of at least %lld bytes required", (long long)need);
     // validate the second stage's arguments before the first stage is enqueued
-    const int64_t d = (int64_t)n_heads * head_dim;
-    CDM_REQUIRE(ldq >= d && ldk >= d && ldv >= d && ldo >= d, CDM_ERR_BAD_ARG, "attn_fwd: row stride smaller than n_heads*head_dim");
+    const int64_t d = (int64_t)n_heads * head_dim, dkv = (int64_t)n_kv_heads * head_dim;
+    CDM_REQUIRE(ldq >= d && ldk >= dkv && ldv >= dkv && ldo >= d, CDM_ERR_BAD_ARG,
+                "attn_fwd: row stride smaller than heads*head_dim");
     CDM_REQUIRE(causal_prefix >= 0 && causal_prefix <= n_tokens, CDM_ERR_BAD_ARG,
                 "attn_fwd: causal_prefix=%lld outside [0, n_tokens]", (long long)causal_prefix);
     CDM_REQUIRE(cdm_aligned16(q) && cdm_aligned16(k) && cdm_aligned16(v) && cdm_aligned16(o) && ldq % 8 == 0 &&
                     ldk % 8 == 0 && ldv % 8 == 0 && ldo % 8 == 0,
                 CDM_ERR_BAD_ALIGN, "attn_fwd: pointers/strides must be 16-byte aligned");
-    if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_heads, head_dim,
+    if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_kv_heads, head_dim,
                                     qk_norm, stream)))
         return rc;
-    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, head_dim, qk_norm, nullptr,
-                                    0, causal_prefix, stream);
+    return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, n_kv_heads, head_dim, qk_norm,
+                                    nullptr, 0, causal_prefix, stream);
 }

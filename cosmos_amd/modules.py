@@ -37,14 +37,16 @@ def _as2d(t: torch.Tensor) -> torch.Tensor:
 class Workspace:
     """Caller-owned scratch tensors of one (n_tokens, d, hidden) shape, reused by every block."""
 
-    def __init__(self, n: int, d: int, hidden: int, n_heads: int, head_dim: int, device):
+    def __init__(self, n: int, d: int, hidden: int, n_heads: int, head_dim: int, device,
+                 n_kv_heads: Optional[int] = None):
         bf = dict(dtype=torch.bfloat16, device=device)
+        n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
         self.n, self.d, self.hidden = n, d, hidden
         self.y = torch.empty((n, d), **bf)
-        self.qkv = torch.empty((n, 3 * d), **bf)
+        self.qkv = torch.empty((n, d + 2 * n_kv_heads * head_dim), **bf)       # [Q | K | V] columns
         self.attn_out = torch.empty((n, d), **bf)
         self.h = torch.empty((n, hidden), **bf)
-        self.attn_ws = torch.empty((max(ops.attn_workspace_bytes(n, n_heads, head_dim), 16),), dtype=torch.uint8,
+        self.attn_ws = torch.empty((max(ops.attn_workspace_bytes(n, n_kv_heads, head_dim), 16),), dtype=torch.uint8,
                                    device=device)
 
     def fits(self, n: int, d: int, hidden: int) -> bool:
@@ -99,23 +101,30 @@ class DMAttnProcessor:
             modality_segments = [(0, n, 0, True)]
         cos, sin = image_rotary_emb
         ws = workspace
-        qkv = ws.qkv if ws is not None else torch.empty((n, 3 * d), dtype=torch.bfloat16, device=x.device)
+        dkv = attn.n_kv_heads * attn.head_dim
+        qkv = ws.qkv if ws is not None else torch.empty((n, d + 2 * dkv), dtype=torch.bfloat16, device=x.device)
+        if qkv.shape[1] != d + 2 * dkv:
+            raise ValueError("workspace was made for another number of K/V heads")
         o = ws.attn_out if ws is not None else torch.empty((n, d), dtype=torch.bfloat16, device=x.device)
 
         wsb = kv_images if kv_images is not None else (ws.attn_ws if ws is not None else None)
-        mask_kw = dict(causal_prefix=causal_prefix, prefix=prefix)
-        q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
+        mask_kw = dict(causal_prefix=causal_prefix, prefix=prefix, n_kv_heads=attn.n_kv_heads)
+        q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
         qkn = attn.qk_norm_args(modality_segments)
         if qkn is not None and self.rope != "in_attention":
             raise NotImplementedError("QK-RMSNorm precedes the rotation: it needs rope='in_attention'")
         if self.rope == "gemm_epilogue":
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
-                         rope_cols=2 * d, head_dim=attn.head_dim)
+                         rope_cols=d + dkv, head_dim=attn.head_dim)
             ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
         else:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
             if self.rope == "streaming":
-                ops.mrope_qk_(q, k, cos, sin, attn.n_heads, attn.head_dim)
+                if attn.n_kv_heads == attn.n_heads:
+                    ops.mrope_qk_(q, k, cos, sin, attn.n_heads, attn.head_dim)
+                else:
+                    ops.mrope_qk_(q, None, cos, sin, attn.n_heads, attn.head_dim)
+                    ops.mrope_qk_(k, None, cos, sin, attn.n_kv_heads, attn.head_dim)
                 ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
             else:     # in registers, inside the attention kernels
                 ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin,
@@ -143,11 +152,15 @@ class DMAttention(nn.Module):
 
     def __init__(self, d_model: int, n_heads: int, head_dim: int, n_branches: int = 1, fp8: bool = False,
                  processor: Optional[DMAttnProcessor] = None, device=None, dtype=torch.bfloat16,
-                 qk_norm: bool = False, eps: float = 1e-6):
+                 qk_norm: bool = False, eps: float = 1e-6, n_kv_heads: Optional[int] = None):
         super().__init__()
         if n_heads * head_dim != d_model:
             raise ValueError("n_heads * head_dim must equal d_model")
+        n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
+        if n_kv_heads < 1 or n_heads % n_kv_heads:
+            raise ValueError("n_kv_heads must divide n_heads")
         self.d_model, self.n_heads, self.head_dim, self.n_branches, self.fp8 = d_model, n_heads, head_dim, n_branches, fp8
+        self.n_kv_heads = n_kv_heads      # K / V heads (num_key_value_heads); fewer than n_heads = grouped-query attention
         kw = dict(device=device, dtype=dtype)
         # per-head QK-RMSNorm weights, one row per branch (norm_q / norm_added_q and norm_k / norm_added_k of the
         # reference's attention layer); fp32 because the kernels normalise in fp32
@@ -157,7 +170,8 @@ class DMAttention(nn.Module):
                                               requires_grad=False)
             self.norm_k_weight = nn.Parameter(torch.ones(n_branches, head_dim, device=device, dtype=torch.float32),
                                               requires_grad=False)
-        self.qkv_weight = nn.ParameterList([nn.Parameter(torch.empty(3 * d_model, d_model, **kw), requires_grad=False)
+        qkv_rows = d_model + 2 * n_kv_heads * head_dim            # rows [Wq | Wk | Wv]
+        self.qkv_weight = nn.ParameterList([nn.Parameter(torch.empty(qkv_rows, d_model, **kw), requires_grad=False)
                                             for _ in range(n_branches)])
         self.out_weight = nn.ParameterList([nn.Parameter(torch.empty(d_model, d_model, **kw), requires_grad=False)
                                             for _ in range(n_branches)])
@@ -228,12 +242,13 @@ class DMBlock(nn.Module):
     """One Mixture-of-Transformers layer (generator side)."""
 
     def __init__(self, d_model: int, n_heads: int, head_dim: int, hidden: int, n_branches: int = 1,
-                 eps: float = 1e-6, fp8: bool = False, device=None, dtype=torch.bfloat16, qk_norm: bool = False):
+                 eps: float = 1e-6, fp8: bool = False, device=None, dtype=torch.bfloat16, qk_norm: bool = False,
+                 n_kv_heads: Optional[int] = None):
         super().__init__()
         kw = dict(device=device, dtype=dtype)
         self.d_model, self.hidden, self.eps, self.fp8, self.n_branches = d_model, hidden, eps, fp8, n_branches
         self.attn = DMAttention(d_model, n_heads, head_dim, n_branches, fp8, device=device, dtype=dtype,
-                                qk_norm=qk_norm, eps=eps)
+                                qk_norm=qk_norm, eps=eps, n_kv_heads=n_kv_heads)
         P = lambda *shape: nn.Parameter(torch.empty(*shape, **kw), requires_grad=False)
         self.norm1_weight = nn.ParameterList([P(d_model) for _ in range(n_branches)])
         self.norm2_weight = nn.ParameterList([P(d_model) for _ in range(n_branches)])
@@ -294,7 +309,7 @@ class DMBlock(nn.Module):
         segs = list(modality_segments) if modality_segments is not None else [(0, n, 0, True)]
         ws = workspace or self._ws
         if ws is None or not ws.fits(n, d, self.hidden) or ws.y.device != x.device:
-            ws = Workspace(n, d, self.hidden, self.attn.n_heads, self.attn.head_dim, x.device)
+            ws = Workspace(n, d, self.hidden, self.attn.n_heads, self.attn.head_dim, x.device, self.attn.n_kv_heads)
             if workspace is None:
                 self._ws = ws
         sh1, sc1, g1, sh2, sc2, g2 = modulation if modulation is not None else self.modulation(temb)
@@ -352,7 +367,8 @@ class DMStack(nn.Module):
         self.cfg = cfg
         self.time_embedder = TimestepEmbedder(cfg.d_model, device=device)
         self.blocks = nn.ModuleList([DMBlock(cfg.d_model, cfg.n_heads, cfg.head_dim, cfg.hidden, cfg.n_branches,
-                                             cfg.eps, cfg.fp8, device=device, dtype=dtype, qk_norm=cfg.qk_norm)
+                                             cfg.eps, cfg.fp8, device=device, dtype=dtype, qk_norm=cfg.qk_norm,
+                                             n_kv_heads=cfg.kv_heads)
                                      for _ in range(cfg.n_blocks)])
         self._rot = None
         self._ws: Optional[Workspace] = None
@@ -407,8 +423,8 @@ class DMStack(nn.Module):
         cos, sin = self.rotary(x.device)
         rot = (cos[:c.n_text].contiguous(), sin[:c.n_text].contiguous())
         segs = [(0, c.n_text, 0, False)]
-        ws = Workspace(c.n_text, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
-        nbytes = ops.attn_workspace_bytes(c.n_text, c.n_heads, c.head_dim)
+        ws = Workspace(c.n_text, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads)
+        nbytes = ops.attn_workspace_bytes(c.n_text, c.kv_heads, c.head_dim)
         images = []
         for blk in self.blocks:
             img = torch.empty((nbytes,), dtype=torch.uint8, device=x.device)
@@ -441,7 +457,7 @@ class DMStack(nn.Module):
         segs = self.segments()
         temb = self.time_embedder(timestep.reshape(-1)[:1])
         if self._ws is None or not self._ws.fits(c.n_tokens, c.d_model, c.hidden) or self._ws.y.device != x.device:
-            self._ws = Workspace(c.n_tokens, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
+            self._ws = Workspace(c.n_tokens, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads)
         for blk in self.blocks:
             blk(x, temb, rot, segs, inplace=True, workspace=self._ws, causal_prefix=c.n_text if c.hybrid_mask else 0)
         video = x[c.n_text:c.n_text + c.n_video]
@@ -471,7 +487,7 @@ class DMStack(nn.Module):
         segs = [(s0 - P, ln, b, m) for (s0, ln, b, m) in self.segments() if s0 >= P]
         temb = self.time_embedder(timestep.reshape(-1)[:1])
         if self._ws_gen is None or not self._ws_gen.fits(n, c.d_model, c.hidden) or self._ws_gen.y.device != x.device:
-            self._ws_gen = Workspace(n, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device)
+            self._ws_gen = Workspace(n, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads)
         for blk, img in zip(self.blocks, cache.images):
             blk(x, temb, self._rot_gen, segs, inplace=True, workspace=self._ws_gen, prefix=(img, P))
         video = x[:c.n_video]

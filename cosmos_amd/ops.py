@@ -273,8 +273,9 @@ def mrope_qk_(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin
     _lib.check(rc, "cdm_mrope_qk_bf16")
 
 
-def attn_workspace_bytes(n_tokens: int, n_heads: int, head_dim: int) -> int:
-    return int(_lib.load().cdm_attn_workspace_bytes(n_tokens, n_heads, head_dim))
+def attn_workspace_bytes(n_tokens: int, n_kv_heads: int, head_dim: int) -> int:
+    """Bytes of the K / V tile images of ``n_tokens`` tokens (``n_kv_heads`` = K / V heads)."""
+    return int(_lib.load().cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim))
 
 
 def _qk_norm_arg(qk_norm, head_dim: int):
@@ -294,7 +295,8 @@ def attention_pack_kv(k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: 
                       workspace: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                       sin: Optional[torch.Tensor] = None, qk_norm=None) -> torch.Tensor:
     """First stage of ``attention``: K (normalised / rotated if asked) and V of ``n`` tokens -> tile images in
-    ``workspace`` (returned).  The images can be kept and passed to ``attention_packed`` as its ``prefix``."""
+    ``workspace`` (returned).  The images can be kept and passed to ``attention_packed`` as its ``prefix``.
+    ``n_heads`` counts K / V heads here (fewer than query heads under grouped-query attention)."""
     lib = _lib.load()
     n, d = k.shape[0], n_heads * head_dim
     if k.shape != (n, d) or v.shape != (n, d):
@@ -314,19 +316,20 @@ def attention_pack_kv(k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: 
 def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, head_dim: int,
                      out: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                      sin: Optional[torch.Tensor] = None, qk_norm=None, prefix=None,
-                     causal_prefix: int = 0) -> torch.Tensor:
+                     causal_prefix: int = 0, n_kv_heads: Optional[int] = None) -> torch.Tensor:
     """Second stage of ``attention``: the ``n`` query rows against the keys packed in ``workspace`` (``n`` tokens),
     preceded by the keys of ``prefix`` = (images, n_prefix_tokens) if given."""
     lib = _lib.load()
     n, d = q.shape[0], n_heads * head_dim
+    n_kv_heads = n_heads if n_kv_heads is None else int(n_kv_heads)
     if out is None:
         out = torch.empty((n, d), dtype=torch.bfloat16, device=q.device)
     half = head_dim // 2
     qn, _keep = _qk_norm_arg(qk_norm, head_dim)
     pws, npre = (None, 0) if prefix is None else (_chk(prefix[0], "prefix images", torch.uint8, 1), int(prefix[1]))
-    if prefix is not None and prefix[0].numel() < attn_workspace_bytes(npre, n_heads, head_dim):
+    if prefix is not None and prefix[0].numel() < attn_workspace_bytes(npre, n_kv_heads, head_dim):
         raise ValueError("prefix images are smaller than the workspace of n_prefix tokens")
-    if workspace.numel() < attn_workspace_bytes(n, n_heads, head_dim):
+    if workspace.numel() < attn_workspace_bytes(n, n_kv_heads, head_dim):
         raise ValueError("workspace is smaller than the images of n tokens")
     timer = _ATTN_TIMER
     if timer is not None:
@@ -334,8 +337,8 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
         e0.record()
     rc = lib.cdm_attn_fwd_packed_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _f32vec(cos, "cos", n * half),
                                       _f32vec(sin, "sin", n * half), _chk(workspace, "workspace", torch.uint8, 1),
-                                      _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, head_dim, qn, pws,
-                                      npre, int(causal_prefix), _stream())
+                                      _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, n_kv_heads, head_dim,
+                                      qn, pws, npre, int(causal_prefix), _stream())
     if timer is not None:
         e1.record()
         timer.append((e0, e1))
@@ -346,8 +349,9 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: int,
               out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
               cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
-              qk_norm=None, causal_prefix: int = 0, prefix=None) -> torch.Tensor:
-    """Attention over the joint sequence; q, k, v: [n, n_heads*head_dim] bf16 views (row stride free).
+              qk_norm=None, causal_prefix: int = 0, prefix=None, n_kv_heads: Optional[int] = None) -> torch.Tensor:
+    """Attention over the joint sequence; q: [n, n_heads*head_dim], k, v: [n, n_kv_heads*head_dim] bf16 views (row
+    stride free; ``n_kv_heads`` defaults to ``n_heads``, fewer = grouped-query attention).
     With cos/sin ([n, head_dim/2] fp32) rotate-half mRoPE is applied to Q and K inside the kernels.
     ``qk_norm`` = (q_weight, k_weight, seg_ends, eps) switches on the per-head RMSNorm of Q and K ahead of the
     rotation: weights [n_seg, head_dim] fp32 on the device, ``seg_ends`` the exclusive end token of each segment.
@@ -356,11 +360,13 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
     lib = _lib.load()
     n = q.shape[0]
     d = n_heads * head_dim
-    if q.shape != (n, d) or k.shape != (n, d) or v.shape != (n, d):
-        raise ValueError("q, k, v must be [n_tokens, n_heads*head_dim]")
+    n_kv_heads = n_heads if n_kv_heads is None else int(n_kv_heads)
+    dkv = n_kv_heads * head_dim
+    if q.shape != (n, d) or k.shape != (n, dkv) or v.shape != (n, dkv):
+        raise ValueError("q must be [n_tokens, n_heads*head_dim] and k, v [n_tokens, n_kv_heads*head_dim]")
     if out is None:
         out = torch.empty((n, d), dtype=torch.bfloat16, device=q.device)
-    need = attn_workspace_bytes(n, n_heads, head_dim)
+    need = attn_workspace_bytes(n, n_kv_heads, head_dim)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
     if _ATTN_TIMER is None and _OP_TIMER is None and prefix is None:
@@ -369,14 +375,14 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
         rc = lib.cdm_attn_fwd_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _chk(k, "k", torch.bfloat16, 2),
                                    k.stride(0), _chk(v, "v", torch.bfloat16, 2), v.stride(0),
                                    _f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half),
-                                   _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, head_dim,
+                                   _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, n_kv_heads, head_dim,
                                    _chk(workspace, "workspace", torch.uint8, 1), workspace.numel(), qn,
                                    int(causal_prefix), _stream())
         _lib.check(rc, "cdm_attn_fwd_bf16")
         return out
     # two-stage form: prefix images, or HIP events around the attention kernel alone while timing is on
-    attention_pack_kv(k, v, n_heads, head_dim, workspace, cos, sin, qk_norm)
-    return attention_packed(q, workspace, n_heads, head_dim, out, cos, sin, qk_norm, prefix, causal_prefix)
+    attention_pack_kv(k, v, n_kv_heads, head_dim, workspace, cos, sin, qk_norm)
+    return attention_packed(q, workspace, n_heads, head_dim, out, cos, sin, qk_norm, prefix, causal_prefix, n_kv_heads)
 
 
 @_timed("step")

@@ -153,21 +153,25 @@ typedef struct cdm_qk_norm {
  * scaled_dot_product_attention (README.md:74; eager form transformers
  * models/qwen3_vl/modeling_qwen3_vl.py:171-193 with fp32 softmax; RoPE :138-142, :412-435).
  *   O = softmax(rope(Q) rope(K)^T / sqrt(head_dim)) V per head, no mask.
- *   q, k, v: [n_tokens, n_heads, head_dim] with row strides ldq, ldk, ldv; o: [n_tokens, n_heads*head_dim] (ldo).
+ *   q: [n_tokens, n_heads, head_dim], k, v: [n_tokens, n_kv_heads, head_dim] with row strides ldq, ldk, ldv;
+ *   o: [n_tokens, n_heads*head_dim] (ldo).  n_kv_heads divides n_heads: query head h uses K / V head
+ *   h / (n_heads / n_kv_heads) (grouped-query attention: num_key_value_heads,
+ *   models/qwen3_vl/configuration_qwen3_vl.py:86; repeat_kv, models/qwen3_vl/modeling_qwen3_vl.py:159-168);
+ *   n_kv_heads = n_heads is plain multi-head attention.
  *   cos, sin: [n_tokens, head_dim/2] fp32 rotary tables, or both null when Q and K are already rotated.
  *   qk_norm: null, or the per-head RMSNorm of Q and K described above.
  *   causal_prefix: 0 = full attention.  P > 0 = the hybrid mask of the architecture figure
  *     (cookbooks/cosmos3/cosmos3-model-architecture.png, right panel; README.md:74): the first P tokens (the AR /
  *     text run) attend causally among themselves and to nothing else, every other token attends to all tokens.
- *   workspace: cdm_attn_workspace_bytes(...) bytes of caller-owned device memory (holds K and V re-laid
- *   out as 64-key tile images); its contents are undefined afterwards.
+ *   workspace: cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim) bytes of caller-owned device memory
+ *   (holds K and V re-laid out as 64-key tile images); its contents are undefined afterwards.
  * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
  */
-int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim);
+int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_kv_heads, int32_t head_dim);
 int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
                           const float* cos, const float* sin, void* o, int64_t ldo, int64_t n_tokens,
-                          int32_t n_heads, int32_t head_dim, void* workspace, int64_t workspace_bytes,
-                          const cdm_qk_norm* qk_norm, int64_t causal_prefix, void* stream);
+                          int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, void* workspace,
+                          int64_t workspace_bytes, const cdm_qk_norm* qk_norm, int64_t causal_prefix, void* stream);
 
 /*
  * The two stages of cdm_attn_fwd_bf16 as separate calls (same operator, same citations): first K (rotated
@@ -179,14 +183,16 @@ int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk
  *   then attend to n_prefix_tokens + n_tokens keys.  Under the hybrid mask the K/V of the text run do not depend on
  *   the denoising step, so they are packed once per prompt and passed here at every step, and the per-step call
  *   carries only the generator tokens.  Cannot be combined with causal_prefix.
+ * cdm_attn_pack_kv_bf16 sees K / V heads only (n_kv_heads of them).
  */
 int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                               const float* sin, void* workspace, int64_t workspace_bytes, int64_t n_tokens,
-                              int32_t n_heads, int32_t head_dim, const cdm_qk_norm* qk_norm, void* stream);
+                              int32_t n_kv_heads, int32_t head_dim, const cdm_qk_norm* qk_norm, void* stream);
 int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, const float* sin,
                                  const void* workspace, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
-                                 int32_t head_dim, const cdm_qk_norm* qk_norm, const void* prefix_workspace,
-                                 int64_t n_prefix_tokens, int64_t causal_prefix, void* stream);
+                                 int32_t n_kv_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
+                                 const void* prefix_workspace, int64_t n_prefix_tokens, int64_t causal_prefix,
+                                 void* stream);
 
 /*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each

@@ -62,17 +62,20 @@ def apply_rope(x, ang):
 
 
 def attention(q, k, v, kv_end=None):
-    """kv_end[n] (optional): query n sees keys 0 .. kv_end[n]-1 only."""
+    """kv_end[n] (optional): query n sees keys 0 .. kv_end[n]-1 only.  k, v may have fewer heads than q
+    (grouped-query attention): query head h then reads K/V head h // (H // Hkv)."""
     N, H, dh = q.shape
+    group = H // k.shape[1]
     o = np.zeros((N, H, dh))
     for h in range(H):
+        g = h // group
         for n in range(N):
             M = k.shape[0] if kv_end is None else int(kv_end[n])
-            sc = np.array([sum(q[n, h, c] * k[m, h, c] for c in range(dh)) for m in range(M)]) / math.sqrt(dh)
+            sc = np.array([sum(q[n, h, c] * k[m, g, c] for c in range(dh)) for m in range(M)]) / math.sqrt(dh)
             e = np.exp(sc - sc.max())
             p = e / e.sum()
             for c in range(dh):
-                o[n, h, c] = sum(p[m] * v[m, h, c] for m in range(M))
+                o[n, h, c] = sum(p[m] * v[m, g, c] for m in range(M))
     return o
 
 

@@ -194,7 +194,9 @@ def hybrid_kv_end(n_tokens: int, causal_prefix: int) -> torch.Tensor:
 
 def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                    kv_end: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Exact attention for a subset of query rows: q_rows[R,H,dh], k,v[N,H,dh] -> [R,H,dh].
+    """Exact attention for a subset of query rows: q_rows[R,H,dh], k,v[N,Hkv,dh] -> [R,H,dh].
+    Hkv divides H: query head h uses K/V head h // (H/Hkv) (grouped-query attention, repeat_kv:
+    TF/models/qwen3_vl/modeling_qwen3_vl.py:159-168,181-182).
 
     softmax(q k^T / sqrt(dh)) v, fp32 softmax
     (TF/models/qwen3_vl/modeling_qwen3_vl.py:171-193; non-causal full
@@ -203,8 +205,7 @@ def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     eager form does with its attention_mask, TF/...modeling_qwen3_vl.py:185-186).
     """
     q = q_rows.to(torch.float32).transpose(0, 1).contiguous()   # [H,R,dh]
-    kk = k.to(torch.float32).transpose(0, 1).contiguous()       # [H,N,dh]
-    vv = v.to(torch.float32).transpose(0, 1).contiguous()
+    kk, vv = _kv_heads(k, q.shape[0]), _kv_heads(v, q.shape[0])   # [H,N,dh]
     s = torch.matmul(q, kk.transpose(1, 2)) * (1.0 / math.sqrt(q.shape[-1]))
     if kv_end is not None:
         hidden = torch.arange(k.shape[0]).view(1, 1, -1) >= kv_end.view(1, -1, 1)
@@ -213,10 +214,20 @@ def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     return torch.matmul(p, vv).transpose(0, 1).contiguous()
 
 
+def _kv_heads(t: torch.Tensor, n_heads: int) -> torch.Tensor:
+    """k or v [N,Hkv,dh] -> [H,N,dh] fp32 with every K/V head repeated H/Hkv times in place (repeat_kv)."""
+    t = t.to(torch.float32).transpose(0, 1).contiguous()
+    if t.shape[0] == n_heads:
+        return t
+    if n_heads % t.shape[0]:
+        raise ValueError("number of K/V heads must divide the number of query heads")
+    return t.repeat_interleave(n_heads // t.shape[0], dim=0)
+
+
 def attention(q, k, v, chunk: int = 1024, kv_end: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Attention, chunked over query rows so scores are never all resident; ``kv_end`` as in attention_rows."""
-    kk = k.to(torch.float32).transpose(0, 1).contiguous()
-    vv = v.to(torch.float32).transpose(0, 1).contiguous()
+    """Attention, chunked over query rows so scores are never all resident; ``kv_end`` and grouped K/V heads as
+    in attention_rows."""
+    kk, vv = _kv_heads(k, q.shape[1]), _kv_heads(v, q.shape[1])
     scale = 1.0 / math.sqrt(q.shape[-1])
     out = []
     for i in range(0, q.shape[0], chunk):
@@ -291,7 +302,8 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
     non-modulated run uses plain RMSNorm and gate 1 (the AR/text branch).
     ``mod`` = (shift1, scale1, gate1, shift2, scale2, gate2), each [d].
     Each weight set: norm1_w, wq, wk, wv, wo, norm2_w, wg, wu, wd ([out, in]);
-    optional norm_q_w / norm_k_w [dh] switch on the per-head QK-RMSNorm.
+    optional norm_q_w / norm_k_w [dh] switch on the per-head QK-RMSNorm.  wk / wv
+    may have fewer rows than wq (n_kv_heads * dh: grouped-query attention).
     ``attn_rows``: optional index tensor; if given only those token rows are
     carried past attention (exact for those rows) and [R, d] is returned.
     """
@@ -300,7 +312,9 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
     dh = d // n_heads
     if segments is None:
         segments = [(0, N, 0, mod is not None)]
-    q = torch.empty(N, d); k = torch.empty(N, d); v = torch.empty(N, d)
+    dkv = weight_sets[segments[0][2]]["wk"].shape[0]
+    n_kv = dkv // dh
+    q = torch.empty(N, d); k = torch.empty(N, dkv); v = torch.empty(N, dkv)
     for (s0, ln, ws, modulated) in segments:
         p = weight_sets[ws]
         sl = slice(s0, s0 + ln)
@@ -309,10 +323,10 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
         q[sl] = _linear(y, p["wq"], fp8); k[sl] = _linear(y, p["wk"], fp8); v[sl] = _linear(y, p["wv"], fp8)
         if "norm_q_w" in p:   # per-head QK-RMSNorm (TF/models/qwen3_vl/modeling_qwen3_vl.py:463-466,479-480)
             q[sl] = rms_norm(q[sl].view(ln, n_heads, dh), p["norm_q_w"], eps).reshape(ln, d)
-            k[sl] = rms_norm(k[sl].view(ln, n_heads, dh), p["norm_k_w"], eps).reshape(ln, d)
+            k[sl] = rms_norm(k[sl].view(ln, n_kv, dh), p["norm_k_w"], eps).reshape(ln, dkv)
     q = apply_mrope(q.view(N, n_heads, dh), cos, sin)
-    k = apply_mrope(k.view(N, n_heads, dh), cos, sin)
-    v = v.view(N, n_heads, dh)
+    k = apply_mrope(k.view(N, n_kv, dh), cos, sin)
+    v = v.view(N, n_kv, dh)
     kv_end = hybrid_kv_end(N, causal_prefix) if causal_prefix else None
     if attn_rows is None:
         o = attention(q, k, v, kv_end=kv_end).reshape(N, d)

@@ -115,6 +115,37 @@ put("ly_wq", a.q_proj.weight); put("ly_wk", a.k_proj.weight); put("ly_wv", a.v_p
 put("ly_norm_q_w", a.q_norm.weight); put("ly_norm_k_w", a.k_norm.weight)
 put("ly_wg", layer.mlp.gate_proj.weight); put("ly_wu", layer.mlp.up_proj.weight); put("ly_wd", layer.mlp.down_proj.weight)
 
+# 8. grouped-query attention (appended last so that the random stream of the sections above is unchanged) -----
+# eager attention with 4 query heads on 2 K/V heads (repeat_kv), and a whole decoder layer with the same grouping
+Hq, Hkv, Ng, dh_g = 4, 2, 19, 32
+q = torch.randn(1, Hq, Ng, dh_g); k = torch.randn(1, Hkv, Ng, dh_g); v = torch.randn(1, Hkv, Ng, dh_g)
+mod = types.SimpleNamespace(num_key_value_groups=Hq // Hkv, training=False)
+o, _ = q3.eager_attention_forward(mod, q, k, v, None, scaling=dh_g ** -0.5)   # [1, N, Hq, dh]
+put("gq_q", q[0]); put("gq_k", k[0]); put("gq_v", v[0]); put("gq_o", o[0])
+
+cfg_g = Qwen3VLTextConfig(hidden_size=Hq * 16, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=16,
+                          intermediate_size=96, hidden_act="silu", num_hidden_layers=1, vocab_size=32, rms_norm_eps=1e-6,
+                          rope_parameters={"rope_type": "default", "rope_theta": 10000.0, "mrope_section": [2, 3, 3],
+                                           "mrope_interleaved": True})
+cfg_g._attn_implementation = "eager"
+layer_g = q3.Qwen3VLTextDecoderLayer(cfg_g, 0).eval()
+with torch.no_grad():
+    for p_ in layer_g.parameters():
+        p_.copy_(torch.randn_like(p_) * (0.2 if p_.ndim == 2 else 1.0))
+rot_g = q3.Qwen3VLTextRotaryEmbedding(cfg_g)
+N_g = 13
+pos_g = torch.stack([torch.randint(0, 30, (N_g,)), torch.randint(0, 9, (N_g,)), torch.randint(0, 9, (N_g,))], 0)
+x = torch.randn(1, N_g, Hq * 16)
+pe = rot_g(x, pos_g[:, None, :])
+with torch.no_grad():
+    y = layer_g(x, position_embeddings=pe, attention_mask=None)
+a = layer_g.self_attn
+put("lg_x", x[0]); put("lg_y", y[0]); put("lg_pos", pos_g); put("lg_sections", [4, 6, 6]); put("lg_heads", Hq)
+put("lg_norm1_w", layer_g.input_layernorm.weight); put("lg_norm2_w", layer_g.post_attention_layernorm.weight)
+put("lg_wq", a.q_proj.weight); put("lg_wk", a.k_proj.weight); put("lg_wv", a.v_proj.weight); put("lg_wo", a.o_proj.weight)
+put("lg_norm_q_w", a.q_norm.weight); put("lg_norm_k_w", a.k_norm.weight)
+put("lg_wg", layer_g.mlp.gate_proj.weight); put("lg_wu", layer_g.mlp.up_proj.weight); put("lg_wd", layer_g.mlp.down_proj.weight)
+
 path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tf_fixtures.npz")
 np.savez_compressed(path, **out)
 print("wrote", path, {k: v.shape for k, v in out.items()})

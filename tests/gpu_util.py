@@ -31,7 +31,8 @@ def oracle_weights(block, branch_count):
     out = []
     for b in range(branch_count):
         qkv = block.attn.qkv_weight[b].detach().float().cpu()
-        out.append(dict(norm1_w=block.norm1_weight[b].detach().float().cpu(), wq=qkv[:d], wk=qkv[d:2 * d], wv=qkv[2 * d:],
+        dkv = getattr(block.attn, "n_kv_heads", block.attn.n_heads) * block.attn.head_dim
+        out.append(dict(norm1_w=block.norm1_weight[b].detach().float().cpu(), wq=qkv[:d], wk=qkv[d:d + dkv], wv=qkv[d + dkv:],
                         wo=block.attn.out_weight[b].detach().float().cpu(),
                         norm2_w=block.norm2_weight[b].detach().float().cpu(),
                         wg=block.gate_weight[b].detach().float().cpu(), wu=block.up_weight[b].detach().float().cpu(),

@@ -47,20 +47,20 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert g(epi=_lib.EPI_GATE_RESIDUAL) == _lib.ERR_BAD_ARG     # R missing
     assert g(epi=_lib.EPI_ROPE_QK) == _lib.ERR_BAD_ARG           # tables missing
     assert g(lda=100) == _lib.ERR_BAD_ARG                        # stride < K
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 48, fake, 1 << 20, None, 0, None) == _lib.ERR_BAD_SHAPE
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 64, fake, 16, None, 0, None) == _lib.ERR_BAD_ARG
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 1, 48, fake, 1 << 20, None, 0, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 1, 64, fake, 16, None, 0, None) == _lib.ERR_BAD_ARG
     assert "workspace" in _lib.last_error()
     assert lib.cdm_mrope_qk_bf16(fake, 64, None, 0, fake, fake, 4, 1, 32, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_quant_rows_e4m3(fake, 128, fake, fake, 4, 100, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_set_variant(b"nope", 0) == _lib.ERR_BAD_ARG
     # empty inputs are accepted without work
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, None, fake, 64, 16, 1, 64, fake, 1 << 20, None, 0, None) == _lib.ERR_BAD_ARG   # cos without sin
-    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 0, 1, 64, None, 0, None, 0, None) == _lib.OK
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, None, fake, 64, 16, 1, 1, 64, fake, 1 << 20, None, 0, None) == _lib.ERR_BAD_ARG   # cos without sin
+    assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 0, 1, 1, 64, None, 0, None, 0, None) == _lib.OK
     # QK-norm descriptor: segments must cover the sequence, 1..8 segments, positive eps, both tables present
     import ctypes as C
     ends = (C.c_int64 * 2)(8, 12)
     qn = _lib.QkNorm(fake, fake, ends, 2, 1e-6)
-    args = (fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 64, fake, 1 << 20)
+    args = (fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 1, 64, fake, 1 << 20)
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG      # covers 12 of 16 tokens
     assert "segments cover" in lib.cdm_last_error().decode()
     qn = _lib.QkNorm(fake, None, ends, 2, 1e-6)
@@ -69,12 +69,21 @@ def test_bad_arguments_are_rejected_on_the_host():
     qn = _lib.QkNorm(fake, fake, ends, 9, 1e-6)
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
     assert lib.cdm_attn_fwd_bf16(*args, None, 17, None) == _lib.ERR_BAD_ARG                  # causal prefix > n_tokens
-    pk = (fake, 64, None, None, fake, fake, 64, 16, 1, 64, None)
+    pk = (fake, 64, None, None, fake, fake, 64, 16, 1, 1, 64, None)
     assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 100, 0, None) == _lib.ERR_BAD_SHAPE       # prefix not whole tiles
     assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 64, 0, None) == _lib.ERR_BAD_ARG          # prefix size without images
     assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 64, 4, None) == _lib.ERR_UNSUPPORTED      # prefix images + causal prefix
     qn = _lib.QkNorm(fake, fake, ends, 2, 0.0)
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
+    # grouped-query attention: the K/V head count must divide the query head count
+    gq = lambda H, Hkv: lib.cdm_attn_fwd_bf16(fake, 64 * H, fake, 64 * max(Hkv, 1), fake, 64 * max(Hkv, 1), None, None, fake,
+                                              64 * H, 16, H, Hkv, 64, fake, 1 << 24, None, 0, None)
+    assert gq(6, 4) == _lib.ERR_BAD_SHAPE and "divide" in _lib.last_error()
+    assert gq(6, 0) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_attn_fwd_packed_bf16(fake, 384, None, None, fake, fake, 384, 16, 6, 4, 64, None, None, 0, 0,
+                                        None) == _lib.ERR_BAD_SHAPE
+    # the workspace holds K/V heads only
+    assert lib.cdm_attn_workspace_bytes(100, 2, 64) * 3 == lib.cdm_attn_workspace_bytes(100, 6, 64)
 
 
 @pytest.mark.skipif(HAS_GPU, reason="needs a host without a GPU")

@@ -30,9 +30,9 @@ def test_attested_key_names_are_classified():
         assert classify(k) is None
 
 
-def small_model(seed):
+def small_model(seed, n_kv_heads=None):
     cfg = DMConfig("ck", 128, 2, 64, 256, 2, (1, 2, 4), n_text=4, n_action=2, n_branches=2, qk_norm=True,
-                   mrope_sections=(16, 24, 24))
+                   mrope_sections=(16, 24, 24), n_kv_heads=n_kv_heads)
     m = DMTransformer(cfg, latent_channels=4, patch=(1, 2, 2), action_dim=6, device="cpu")
     g = torch.Generator().manual_seed(seed)
     with torch.no_grad():
@@ -66,6 +66,23 @@ def test_safetensors_round_trip(tmp_path):
     bad["layers.0.self_attn.add_q_proj.weight"] = torch.zeros(5, 5)
     with pytest.raises(ValueError):
         load_generator_weights(small_model(4), bad)
+
+
+def test_round_trip_with_grouped_kv_heads():
+    """One K/V head for two query heads: k_proj / v_proj have d_kv = 64 rows and land behind the 128 q rows."""
+    a, b = small_model(6, n_kv_heads=1), small_model(7, n_kv_heads=1)
+    sd = export_generator_weights(a)
+    assert sd["layers.0.self_attn.add_q_proj.weight"].shape == (128, 128)
+    assert sd["layers.0.self_attn.add_k_proj.weight"].shape == (64, 128)
+    assert sd["layers.0.self_attn.to_v.weight"].shape == (64, 128)
+    w = a.stack.blocks[0].attn.qkv_weight[1]
+    assert w.shape == (256, 128) and torch.equal(sd["layers.0.self_attn.add_v_proj.weight"], w[192:])
+    rep = load_generator_weights(b, sd)
+    assert rep["missing"] == [] and rep["unexpected"] == []
+    for (na, pa), (nb, pb) in zip(a.named_parameters(), b.named_parameters()):
+        assert na == nb and torch.equal(pa, pb), na
+    with pytest.raises(ValueError):      # a multi-head checkpoint does not fit a grouped-query model
+        load_generator_weights(small_model(8, n_kv_heads=1), export_generator_weights(small_model(9)))
 
 
 def test_patchify_round_trip_and_order():

@@ -111,9 +111,12 @@ def test_mot_three_branch_block():
     assert_close(y3, y1.float().cpu(), 0.99999, 2e-3, "equal weights == single branch")
 
 
-def test_mot_block_with_qk_norm():
-    """Three-branch block with the per-head QK-RMSNorm switched on (own weight row per branch)."""
-    cfg = DMConfig("motn", 256, 2, 128, 512, 1, (2, 4, 8), n_text=40, n_action=24, n_branches=3, qk_norm=True)
+@pytest.mark.parametrize("n_kv_heads", [None, 1])
+def test_mot_block_with_qk_norm(n_kv_heads):
+    """Three-branch block with the per-head QK-RMSNorm switched on (own weight row per branch); with one K/V head
+    for the two query heads as well (grouped-query attention: the fused QKV weight then has d + 2 d_kv rows)."""
+    cfg = DMConfig("motn", 256, 2, 128, 512, 1, (2, 4, 8), n_text=40, n_action=24, n_branches=3, qk_norm=True,
+                   n_kv_heads=n_kv_heads)
     st = DMStack(cfg, device=dev())
     blk = st.blocks[0]
     g = torch.Generator(device=dev()).manual_seed(21)

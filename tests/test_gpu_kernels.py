@@ -287,6 +287,35 @@ def test_attention_hybrid_mask(n, P, H, hd, variant):
     assert_close(o[:1], qkvr[:1, 2 * d:], 0.99999, 5e-3, "first token sees only itself")
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n,H,Hkv,hd,P", [(300, 8, 2, 128, 0), (257, 6, 3, 64, 0), (200, 4, 1, 128, 70), (1100, 16, 4, 64, 0),
+                                          (513, 12, 12, 64, 0)])
+def test_attention_grouped_query(n, H, Hkv, hd, P, variant, request):
+    """n_kv_heads < n_heads: query head h reads K/V head h // (H / Hkv); with mRoPE and QK-norm in registers and
+    (P > 0) the hybrid mask.  12 heads also puts two heads on some XCDs and one on others."""
+    prev = ops.set_variant("attn", variant)
+    request.addfinalizer(lambda: ops.set_variant("attn", prev))
+    g = gen(n + H + 7 * Hkv)
+    d, dkv = H * hd, Hkv * hd
+    pos, _ = rotary.build_positions(n, (0, 0, 0), 0)
+    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48) if hd == 128 else (16, 24, 24))
+    qkv, qkvr = rand_bf16((n, d + 2 * dkv), g, 1.5)
+    qw, kw = 1 + 0.3 * torch.randn(1, hd, generator=g), 1 + 0.3 * torch.randn(1, hd, generator=g)
+    q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
+    o = ops.attention(q, k, v, H, hd, cos=cos.to(dev()), sin=sin.to(dev()), qk_norm=(qw.to(dev()), kw.to(dev()), [n], 1e-6),
+                      causal_prefix=P, n_kv_heads=Hkv)
+    qn = O.apply_mrope(O.rms_norm(qkvr[:, :d].view(n, H, hd), qw[0], 1e-6), cos, sin)
+    kn = O.apply_mrope(O.rms_norm(qkvr[:, d:d + dkv].view(n, Hkv, hd), kw[0], 1e-6), cos, sin)
+    want = O.attention(qn, kn, qkvr[:, d + dkv:].view(n, Hkv, hd), kv_end=O.hybrid_kv_end(n, P) if P else None)
+    assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"GQA attention n={n} H={H}/{Hkv} hd={hd} P={P} variant={variant}")
+    if Hkv < H:
+        # same result as multi-head attention on K/V whose heads were repeated in memory
+        rep = lambda t: t.view(n, Hkv, 1, hd).expand(n, Hkv, H // Hkv, hd).reshape(n, d).contiguous()
+        o2 = ops.attention(q, rep(k), rep(v), H, hd, cos=cos.to(dev()), sin=sin.to(dev()),
+                           qk_norm=(qw.to(dev()), kw.to(dev()), [n], 1e-6), causal_prefix=P)
+        assert torch.equal(o, o2)
+
+
 @pytest.mark.parametrize("P,m,H,hd", [(64, 200, 2, 128), (128, 65, 1, 64), (512, 700, 1, 128)])
 def test_attention_with_prefix_key_images(P, m, H, hd):
     """Keys packed once (the text run) and prepended to the per-call keys: the m query rows must equal rows P.. of

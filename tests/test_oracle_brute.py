@@ -221,3 +221,18 @@ def test_hybrid_mask_attention():
     # ... and equal the block run on the prefix alone with a causal mask
     y3 = O.dm_block(x[:P], [w], mod, cos[:P], sin[:P], H, [(0, P, 0, False)], causal_prefix=P)
     assert torch.allclose(y[:P], y3, atol=1e-5)
+
+
+def test_grouped_query_attention_brute_and_equivalence():
+    """Grouped K/V heads: against the float64 brute force (with the hybrid mask on top), and against plain
+    multi-head attention on K/V whose heads were repeated by hand."""
+    g = torch.Generator().manual_seed(13)
+    N, H, Hkv, dh = 9, 6, 2, 8
+    q = torch.randn(N, H, dh, generator=g)
+    k, v = (torch.randn(N, Hkv, dh, generator=g) for _ in range(2))
+    kv_end = O.hybrid_kv_end(N, 3)
+    got = O.attention(q, k, v, chunk=4, kv_end=kv_end)
+    want = B.attention(q.double().numpy(), k.double().numpy(), v.double().numpy(), kv_end.numpy())
+    assert np.abs(got.double().numpy() - want).max() < 1e-5
+    rep = lambda t: torch.stack([t[:, h // (H // Hkv)] for h in range(H)], dim=1)
+    assert torch.allclose(O.attention(q, k, v), O.attention(q, rep(k), rep(v)), atol=1e-6)

@@ -76,3 +76,24 @@ def test_unmodulated_block_wiring_against_decoder_layer(golden):
     # row-sampled form is exact for the sampled rows
     rows = torch.tensor([0, 5, 11])
     close(O.dm_block(T(g["ly_x"]), [w], None, cos, sin, H, attn_rows=rows), g["ly_y"][[0, 5, 11]], 2e-5)
+
+
+def test_grouped_query_attention(golden):
+    """4 query heads on 2 K/V heads against the library's eager attention (repeat_kv)."""
+    q, k, v = (T(golden[n]).transpose(0, 1) for n in ("gq_q", "gq_k", "gq_v"))   # [N,Hq,dh], [N,Hkv,dh]
+    assert q.shape[1] == 4 and k.shape[1] == 2
+    close(O.attention(q, k, v, chunk=7), golden["gq_o"], 1e-5)
+    close(O.attention_rows(q[[0, 9, 18]], k, v), golden["gq_o"][[0, 9, 18]], 1e-5)
+    # a wrong head pairing (interleaved instead of blocked repetition) is a different function
+    wrong = O.attention(q, k.flip(1), v.flip(1))
+    assert float((wrong - T(golden["gq_o"])).abs().max()) > 1e-2
+
+
+def test_grouped_query_block_wiring_against_decoder_layer(golden):
+    g = golden
+    w = {k: T(g["lg_" + k]) for k in ("norm1_w", "norm2_w", "wq", "wk", "wv", "wo", "wg", "wu", "wd",
+                                       "norm_q_w", "norm_k_w")}
+    H = int(g["lg_heads"]); d = g["lg_x"].shape[1]
+    assert w["wk"].shape[0] * 2 == w["wq"].shape[0]
+    cos, sin = O.mrope_cos_sin(T(g["lg_pos"]), d // H, [int(s) for s in g["lg_sections"]], 10000.0, "interleaved")
+    close(O.dm_block(T(g["lg_x"]), [w], None, cos, sin, H), g["lg_y"], 2e-5)
