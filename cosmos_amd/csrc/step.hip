@@ -6,23 +6,25 @@
 namespace {
 
 constexpr int kMaxHist = 4;
+constexpr int kMaxOut = 3;
 
 struct StepParams {
     const float* x;
     const bf16_t* vc;
     const bf16_t* vu;          // null = no guidance (v = vc)
     const float* hist[kMaxHist];
-    float c_x, c_v, c_h[kMaxHist];
-    int n_hist;
+    float c[kMaxOut][2 + kMaxHist];      // row j: coefficients of output j for (x, v, hist[0..])
+    float* out[kMaxOut];
+    int n_hist, n_out;
     float guidance;
-    float* v_out;              // null or the combined prediction (fp32), the next call's history
-    float* out;
     int64_t n;
 };
 
 __device__ __forceinline__ float combine(float c, float u, float g, bool guided) { return guided ? u + g * (c - u) : c; }
 
-// 4 elements per thread per iteration: 8-byte loads of the bf16 predictions, 16-byte loads/stores of the fp32 tensors
+// 4 elements per thread per iteration: 8-byte loads of the bf16 predictions, 16-byte loads/stores of the fp32 tensors.
+// Every input element is read before any output element of the same index is written and elements are independent,
+// so an output may be the very tensor of an input (the latents in place, a history slot being recycled).
 __global__ __launch_bounds__(256) void cfg_step_kernel(const StepParams p) {
     const bool guided = p.vu != nullptr;
     const int64_t n4 = p.n >> 2;
@@ -31,18 +33,30 @@ __global__ __launch_bounds__(256) void cfg_step_kernel(const StepParams p) {
         uint2 u2 = c2;
         if (guided) u2 = reinterpret_cast<const uint2*>(p.vu)[i];
         const float4 x4 = reinterpret_cast<const float4*>(p.x)[i];
-        float v[4] = {combine(bf16lo(c2.x), bf16lo(u2.x), p.guidance, guided), combine(bf16hi(c2.x), bf16hi(u2.x), p.guidance, guided),
-                      combine(bf16lo(c2.y), bf16lo(u2.y), p.guidance, guided), combine(bf16hi(c2.y), bf16hi(u2.y), p.guidance, guided)};
-        float o[4] = {p.c_x * x4.x + p.c_v * v[0], p.c_x * x4.y + p.c_v * v[1], p.c_x * x4.z + p.c_v * v[2],
-                      p.c_x * x4.w + p.c_v * v[3]};
+        const float x[4] = {x4.x, x4.y, x4.z, x4.w};
+        const float v[4] = {combine(bf16lo(c2.x), bf16lo(u2.x), p.guidance, guided), combine(bf16hi(c2.x), bf16hi(u2.x), p.guidance, guided),
+                            combine(bf16lo(c2.y), bf16lo(u2.y), p.guidance, guided), combine(bf16hi(c2.y), bf16hi(u2.y), p.guidance, guided)};
+        float h[kMaxHist][4];
 #pragma unroll
-        for (int h = 0; h < kMaxHist; ++h)
-            if (h < p.n_hist) {
-                const float4 h4 = reinterpret_cast<const float4*>(p.hist[h])[i];
-                o[0] += p.c_h[h] * h4.x; o[1] += p.c_h[h] * h4.y; o[2] += p.c_h[h] * h4.z; o[3] += p.c_h[h] * h4.w;
+        for (int k = 0; k < kMaxHist; ++k)
+            if (k < p.n_hist) {
+                const float4 h4 = reinterpret_cast<const float4*>(p.hist[k])[i];
+                h[k][0] = h4.x; h[k][1] = h4.y; h[k][2] = h4.z; h[k][3] = h4.w;
             }
-        if (p.v_out) reinterpret_cast<float4*>(p.v_out)[i] = make_float4(v[0], v[1], v[2], v[3]);
-        reinterpret_cast<float4*>(p.out)[i] = make_float4(o[0], o[1], o[2], o[3]);
+#pragma unroll
+        for (int j = 0; j < kMaxOut; ++j)
+            if (j < p.n_out) {
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = p.c[j][0] * x[e] + p.c[j][1] * v[e];
+#pragma unroll
+                for (int k = 0; k < kMaxHist; ++k)
+                    if (k < p.n_hist) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] += p.c[j][2 + k] * h[k][e];
+                    }
+                reinterpret_cast<float4*>(p.out[j])[i] = make_float4(o[0], o[1], o[2], o[3]);
+            }
     }
     // tail (n % 4 elements), one thread each
     const int64_t t = (n4 << 2) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -50,34 +64,42 @@ __global__ __launch_bounds__(256) void cfg_step_kernel(const StepParams p) {
         const float c = bf16_bits_to_f32(p.vc[t]);
         const float u = guided ? bf16_bits_to_f32(p.vu[t]) : c;
         const float v = combine(c, u, p.guidance, guided);
-        float o = p.c_x * p.x[t] + p.c_v * v;
-        for (int h = 0; h < p.n_hist; ++h) o += p.c_h[h] * p.hist[h][t];
-        if (p.v_out) p.v_out[t] = v;
-        p.out[t] = o;
+        const float x = p.x[t];
+        float h[kMaxHist];
+        for (int k = 0; k < p.n_hist; ++k) h[k] = p.hist[k][t];
+        for (int j = 0; j < p.n_out; ++j) {
+            float o = p.c[j][0] * x + p.c[j][1] * v;
+            for (int k = 0; k < p.n_hist; ++k) o += p.c[j][2 + k] * h[k];
+            p.out[j][t] = o;
+        }
     }
 }
 
 }  // namespace
 
 extern "C" int32_t cdm_cfg_step_f32(const float* x, const void* v_cond, const void* v_uncond, float guidance,
-                                    const float* const* hist, const float* coef, int32_t n_hist, float* v_out,
-                                    float* out, int64_t n, void* stream) {
-    CDM_REQUIRE(x && v_cond && out && coef, CDM_ERR_BAD_ARG, "cfg_step: null pointer");
+                                    const float* const* hist, int32_t n_hist, const float* coef, float* const* outs,
+                                    int32_t n_out, int64_t n, void* stream) {
+    CDM_REQUIRE(x && v_cond && outs && coef, CDM_ERR_BAD_ARG, "cfg_step: null pointer");
     CDM_REQUIRE(n >= 0, CDM_ERR_BAD_ARG, "cfg_step: negative size");
     CDM_REQUIRE(n_hist >= 0 && n_hist <= kMaxHist, CDM_ERR_BAD_ARG, "cfg_step: n_hist=%d must be 0..%d", n_hist, kMaxHist);
+    CDM_REQUIRE(n_out >= 1 && n_out <= kMaxOut, CDM_ERR_BAD_ARG, "cfg_step: n_out=%d must be 1..%d", n_out, kMaxOut);
     CDM_REQUIRE(n_hist == 0 || hist, CDM_ERR_BAD_ARG, "cfg_step: history pointers missing");
-    CDM_REQUIRE(cdm_aligned16(x) && cdm_aligned16(v_cond) && cdm_aligned16(v_uncond) && cdm_aligned16(out) &&
-                    cdm_aligned16(v_out),
-                CDM_ERR_BAD_ALIGN, "cfg_step: pointers must be 16-byte aligned");
+    CDM_REQUIRE(cdm_aligned16(x) && cdm_aligned16(v_cond) && cdm_aligned16(v_uncond), CDM_ERR_BAD_ALIGN,
+                "cfg_step: pointers must be 16-byte aligned");
     StepParams p{};
     p.x = x; p.vc = (const bf16_t*)v_cond; p.vu = (const bf16_t*)v_uncond;
-    p.c_x = coef[0]; p.c_v = coef[1];
     for (int h = 0; h < n_hist; ++h) {
         CDM_REQUIRE(hist[h] && cdm_aligned16(hist[h]), CDM_ERR_BAD_ARG, "cfg_step: history tensor %d null or misaligned", h);
         p.hist[h] = hist[h];
-        p.c_h[h] = coef[2 + h];
     }
-    p.n_hist = n_hist; p.guidance = guidance; p.v_out = v_out; p.out = out; p.n = n;
+    for (int j = 0; j < n_out; ++j) {
+        CDM_REQUIRE(outs[j] && cdm_aligned16(outs[j]), CDM_ERR_BAD_ARG, "cfg_step: output tensor %d null or misaligned", j);
+        for (int k = 0; k < j; ++k) CDM_REQUIRE(outs[j] != outs[k], CDM_ERR_BAD_ARG, "cfg_step: outputs %d and %d coincide", k, j);
+        p.out[j] = outs[j];
+        for (int k = 0; k < 2 + n_hist; ++k) p.c[j][k] = coef[j * (2 + n_hist) + k];
+    }
+    p.n_hist = n_hist; p.n_out = n_out; p.guidance = guidance; p.n = n;
     if (n == 0) return CDM_OK;
     int32_t rc = cdm_require_device();
     if (rc) return rc;

@@ -386,32 +386,44 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
 
 
 @_timed("step")
-def cfg_step(x: torch.Tensor, v_cond: torch.Tensor, v_uncond: Optional[torch.Tensor], guidance: float,
-             coef: Sequence[float], hist: Sequence[torch.Tensor] = (), v_out: Optional[torch.Tensor] = None,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = coef[0] x + coef[1] v + sum_i coef[2+i] hist[i], v = v_uncond + guidance (v_cond - v_uncond)
-    (v = v_cond without v_uncond).  x, out, hist, v_out: fp32; v_cond, v_uncond: bf16; all of one shape, contiguous.
-    ``out`` may be ``x`` itself."""
+def cfg_multistep(x: torch.Tensor, v_cond: torch.Tensor, v_uncond: Optional[torch.Tensor], guidance: float,
+                  coef: Sequence[Sequence[float]], hist: Sequence[torch.Tensor], outs: Sequence[torch.Tensor]) -> None:
+    """outs[j] = coef[j][0] x + coef[j][1] v + sum_k coef[j][2+k] hist[k] with v = v_uncond + guidance (v_cond -
+    v_uncond) (v = v_cond without v_uncond), all outputs in ONE pass.  x, hist, outs: fp32; v_cond, v_uncond: bf16; all
+    of one shape, contiguous.  An output may be ``x`` or one of ``hist`` (in place)."""
     lib = _lib.load()
     n = x.numel()
-    if len(coef) != 2 + len(hist):
-        raise ValueError("coef must hold 2 + len(hist) values")
+    if not 1 <= len(outs) <= 3 or len(coef) != len(outs) or any(len(r) != 2 + len(hist) for r in coef):
+        raise ValueError("coef must have one row of 2 + len(hist) values per output (1..3 outputs)")
     for t, name, dt in [(x, "x", torch.float32), (v_cond, "v_cond", torch.bfloat16)] + \
                        ([(v_uncond, "v_uncond", torch.bfloat16)] if v_uncond is not None else []) + \
-                       [(h, "hist", torch.float32) for h in hist] + \
-                       ([(v_out, "v_out", torch.float32)] if v_out is not None else []):
+                       [(h, "hist", torch.float32) for h in hist] + [(o, "out", torch.float32) for o in outs]:
         if t.numel() != n or not t.is_contiguous():
             raise ValueError(f"{name} must be contiguous with {n} elements")
         _chk(t.reshape(-1), name, dt)
+    hp = (C.c_void_p * max(len(hist), 1))(*[h.data_ptr() for h in hist])
+    op = (C.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
+    flat = [float(c) for row in coef for c in row]
+    cf = (C.c_float * len(flat))(*flat)
+    rc = lib.cdm_cfg_step_f32(x.data_ptr(), v_cond.data_ptr(), v_uncond.data_ptr() if v_uncond is not None else None,
+                              float(guidance), hp, len(hist), cf, op, len(outs), n, _stream())
+    _lib.check(rc, "cdm_cfg_step_f32")
+
+
+def cfg_step(x: torch.Tensor, v_cond: torch.Tensor, v_uncond: Optional[torch.Tensor], guidance: float,
+             coef: Sequence[float], hist: Sequence[torch.Tensor] = (), v_out: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = coef[0] x + coef[1] v + sum_i coef[2+i] hist[i]; ``v_out`` (optional) receives the guided prediction v.
+    ``out`` may be ``x`` itself.  The single-update form of ``cfg_multistep``."""
+    if len(coef) != 2 + len(hist):
+        raise ValueError("coef must hold 2 + len(hist) values")
     if out is None:
         out = torch.empty_like(x)
-    _chk(out.reshape(-1), "out", torch.float32)
-    hp = (C.c_void_p * max(len(hist), 1))(*[h.data_ptr() for h in hist])
-    cf = (C.c_float * len(coef))(*[float(c) for c in coef])
-    rc = lib.cdm_cfg_step_f32(x.data_ptr(), v_cond.data_ptr(), v_uncond.data_ptr() if v_uncond is not None else None,
-                              float(guidance), hp, cf, len(hist), v_out.data_ptr() if v_out is not None else None,
-                              out.data_ptr(), n, _stream())
-    _lib.check(rc, "cdm_cfg_step_f32")
+    rows, outs = [list(coef)], [out]
+    if v_out is not None:
+        rows.append([0.0, 1.0] + [0.0] * len(hist))
+        outs.append(v_out)
+    cfg_multistep(x, v_cond, v_uncond, guidance, rows, hist, outs)
     return out
 
 

@@ -230,17 +230,21 @@ int32_t cdm_set_variant(const char* op, int32_t variant);
  * Classifier-free-guidance combine fused with the scheduler's linear latent update - replaces, inside one
  * denoising iteration of the pipeline (Cosmos3OmniPipeline.__call__, README.md:249-263: guidance_scale;
  * README.md:247: UniPCMultistepScheduler with flow_shift), the elementwise tail
- *     v   = v_uncond + guidance * (v_cond - v_uncond)            (v = v_cond when v_uncond is null)
- *     out = coef[0] * x + coef[1] * v + sum_i coef[2 + i] * hist[i]
- * which is the form of an Euler flow-matching step (coef = {1, sigma_next - sigma}) and of every linear multistep
- * update (UniPC, DPM-Solver++): the scheduler computes the scalar coefficients on the host, this kernel makes one
- * pass over the tensors.  x, out, hist[i], v_out: fp32 [n]; v_cond, v_uncond: bf16 [n] (the transformer's output);
- * v_out (optional) receives v, the model output a multistep scheduler keeps as history; out may alias x.
- * hist and coef are HOST arrays (n_hist <= 4 device pointers; 2 + n_hist floats).
+ *     v       = v_uncond + guidance * (v_cond - v_uncond)            (v = v_cond when v_uncond is null)
+ *     outs[j] = coef[j][0] * x + coef[j][1] * v + sum_k coef[j][2 + k] * hist[k]        j = 0 .. n_out-1
+ * which is the form of an Euler flow-matching step (one output, coef = {1, sigma_next - sigma}) and of every linear
+ * multistep update: a UniPC step (corrector of the current latents, then predictor) is three outputs - the next
+ * latents, the corrected latents the next corrector starts from, and the data prediction x - sigma v kept as
+ * history - of the current latents, the prediction, the previous corrected latents and the kept data predictions.
+ * The scheduler computes the scalar coefficients on the host; this kernel makes ONE pass over the tensors.
+ *   x, hist[k], outs[j]: fp32 [n]; v_cond, v_uncond: bf16 [n] (the transformer's output).
+ *   hist, outs: HOST arrays of n_hist (0..4) / n_out (1..3) device pointers; coef: HOST array, row-major
+ *   [n_out][2 + n_hist].  An output may be x or a hist tensor itself (in-place latents, a recycled history slot);
+ *   two outputs may not coincide.
  */
 int32_t cdm_cfg_step_f32(const float* x, const void* v_cond, const void* v_uncond, float guidance,
-                         const float* const* hist, const float* coef, int32_t n_hist, float* v_out, float* out,
-                         int64_t n, void* stream);
+                         const float* const* hist, int32_t n_hist, const float* coef, float* const* outs,
+                         int32_t n_out, int64_t n, void* stream);
 
 #ifdef __cplusplus
 }

@@ -19,19 +19,23 @@ Pinning status of each oracle function
 pinned by library golden vectors (tests/golden/tf_fixtures.npz) and by
 closed forms / float64 brute force (tests/test_oracle_*.py):
     rms_norm, rotate-half mRoPE (chunked and interleaved tables, apply),
-    vision / text position ids, attention, swiglu, pre-norm residual wiring.
+    vision / text position ids, attention (multi-head and grouped-query),
+    swiglu, pre-norm residual wiring (also with grouped K/V heads).
 pinned by closed forms and float64 brute force only (no library routine
 exists for them):
     adaln_rms_norm modulation, gated residual, MoT segment routing,
     e4m3 quantisation (against torch.float8_e4m3fn casts), cfg_step (guidance
-    combine + linear scheduler update).
+    combine + linear scheduler update); oracle/unipc.py (UniPC predictor /
+    corrector updates: Euler closed form, exactness on polynomial data
+    predictions against quadrature of the exact solution, convergence orders).
 parity unpinned against the real Cosmos 3 generator (only an import of the
 absent diffusers implementation could pin them; the benchmark configuration
 text governs instead):
     timestep_embedding / time_mlp conventions, adaLN chunk order and the
     (1 + scale) convention, mRoPE channel layout choice (chunked is the
     default), modality position offsets in generator mode, the fp8 recipe,
-    the scheduler's coefficient rule (flow_sigmas is the plain shifted Euler
-    schedule; the reference's UniPC coefficients live in diffusers).
+    the scheduler as diffusers configures it (oracle/unipc.py restates the
+    published UniPC algorithm; diffusers' noise-level grid, default order and
+    final-step handling are restated from its documentation, not executed).
 """
 from .dm_oracle import *  # noqa: F401,F403

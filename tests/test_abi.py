@@ -86,6 +86,22 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_workspace_bytes(100, 2, 64) * 3 == lib.cdm_attn_workspace_bytes(100, 6, 64)
 
 
+def test_step_arguments_are_validated_on_the_host():
+    lib = _lib.load()
+    fake = 0x10000
+    coef = (C.c_float * 6)(1, 1, 0, 1, 1, 0)
+    outs = (C.c_void_p * 2)(fake, fake + 64)
+    hist = (C.c_void_p * 1)(fake + 128)
+    call = lambda n_hist=1, n_out=2, outs=outs: lib.cdm_cfg_step_f32(fake, fake, None, 1.0, hist, n_hist, coef, outs, n_out, 0, None)
+    assert call() == _lib.OK                                   # n = 0: accepted without work
+    assert call(n_out=0) == _lib.ERR_BAD_ARG and call(n_out=4) == _lib.ERR_BAD_ARG
+    assert call(n_hist=5) == _lib.ERR_BAD_ARG
+    same = (C.c_void_p * 2)(fake, fake)
+    assert call(outs=same) == _lib.ERR_BAD_ARG and "coincide" in _lib.last_error()
+    odd = (C.c_void_p * 2)(fake, fake + 4)
+    assert call(outs=odd) == _lib.ERR_BAD_ARG
+
+
 @pytest.mark.skipif(HAS_GPU, reason="needs a host without a GPU")
 def test_valid_call_without_a_device_reports_no_device():
     lib = _lib.load()
