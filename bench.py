@@ -113,7 +113,7 @@ def main():
     ap.add_argument("--attn-variant", type=int, default=0)
     ap.add_argument("--gemm-variant", type=int, default=0)
     ap.add_argument("--rope", default="in_attention", choices=["in_attention", "gemm_epilogue", "streaming"])
-    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="counter calibration aid: after the timed region run ONE plain streaming kernel that reads and "
