@@ -1,4 +1,6 @@
-// Non-causal full self-attention (flash-style, online softmax) on the gfx950 matrix cores.
+// Full self-attention over the joint sequence (flash-style, online softmax) on the gfx950 matrix cores; optional
+// hybrid mask (a causal prefix that is blind to the rest), grouped K / V heads, prefix key images packed by an
+// earlier call, per-head RMSNorm of Q and K.
 //
 // Work split: one workgroup owns 256 query rows of one head and streams all keys in tiles of 64.
 // Scores are computed TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_32x32x16_bf16: the A operand is a K
@@ -9,8 +11,8 @@
 // operand of O^T += V^T . P^T, whose A operand is a row of V^T.  The K rows of a 32-key block are
 // fetched in a permuted order so that the 8 keys a lane holds in accumulator registers 8j..8j+7 are
 // the 8 consecutive keys the second product expects.
-// Rotate-half mRoPE is applied in registers: to K while it is re-tiled for the kernel, to Q when the
-// kernel loads its Q fragments (both members of a rotary pair sit in the same lane).
+// Rotate-half mRoPE (and the QK-RMSNorm ahead of it) is applied in registers: to K while it is re-tiled for the
+// kernel, to Q when the kernel loads its Q fragments (both members of a rotary pair sit in the same lane).
 #include "cdm_common.h"
 
 namespace {
