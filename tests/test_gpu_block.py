@@ -303,12 +303,14 @@ def test_transformer_with_stack_edges_and_loaded_checkpoint(tmp_path):
     assert_close(out["action"][0], want_act, BF16_COS, BF16_REL, "action head")
 
 
-def test_hybrid_mask_stack_and_context_reuse():
+@pytest.mark.parametrize("n_kv_heads", [None, 1])
+def test_hybrid_mask_stack_and_context_reuse(n_kv_heads):
     """Two-branch stack under the hybrid mask: (1) joint forward vs the masked fp32 oracle; (2) the text run's K/V
     packed once per prompt and reused: same video output from a forward that carries only the generator tokens;
-    (3) the reused cache stays valid for another timestep."""
+    (3) the reused cache stays valid for another timestep.  Also with one K/V head for the two query heads (the kept
+    images then hold K/V heads only)."""
     cfg = DMConfig("hyb", 256, 2, 128, 512, 2, (2, 5, 8), n_text=64, n_action=7, n_branches=3, qk_norm=True,
-                   hybrid_mask=True)
+                   hybrid_mask=True, n_kv_heads=n_kv_heads)
     st = DMStack(cfg, device=dev())
     st.reset_parameters(41)
     g = torch.Generator(device=dev()).manual_seed(41)
