@@ -191,7 +191,13 @@ __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, con
         const int rloc = it * RPI + rl;
         const uint4 v = *reinterpret_cast<const uint4*>(stage + rloc * kStagePitch + ch * 16);
         const int row = row0 + rloc;
-        if (row < t.m_end && col < p.N) *reinterpret_cast<uint4*>(p.C + (int64_t)row * p.ldc + col) = v;
+        // non-temporal: the output is not read again by this kernel, and a tile's 128 KB per CU (4 MB per XCD at a
+        // time, the whole L2) would otherwise push the A / W slabs of the next tiles out of the cache
+        if (row < t.m_end && col < p.N) {
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            const u32x4 vv = {v.x, v.y, v.z, v.w};
+            __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(p.C + (int64_t)row * p.ldc + col));
+        }
     }
 }
 
