@@ -417,3 +417,102 @@ def test_gemm_fp8(M, N, K, epi, variant, request):
     # against the UNQUANTISED product the error is the e4m3 quantisation noise itself (K is only 256-512 here and
     # SWIGLU multiplies two quantised products); the 5e-2 / 0.999 bar is checked on whole blocks in test_gpu_block
     assert_close(c, ref32, 0.997, 8e-2, f"fp8 gemm vs fp32 ({epi})")
+
+
+# ------------------------------------------------------------------ seeded sweeps over valid shapes
+def _sweep(seed, count):
+    import random
+    rnd = random.Random(seed)
+    return [rnd.randrange(1 << 30) for _ in range(count)]
+
+
+@pytest.mark.parametrize("case", _sweep(20250, 20))
+def test_attention_shape_sweep(case):
+    """Random valid combinations of sequence length (ragged tiles and query blocks), head counts (not multiples of the
+    8 XCDs), K/V grouping, head size, causal prefix, rotary tables and QK-norm segments against the oracle."""
+    import random
+    rnd = random.Random(case)
+    hd = rnd.choice([64, 128])
+    Hkv = rnd.choice([1, 2, 3, 5])
+    H = Hkv * rnd.choice([1, 1, 2, 4])
+    n = rnd.choice([rnd.randrange(1, 130), rnd.randrange(130, 700), rnd.randrange(700, 1500)])
+    P = rnd.choice([0, 0, rnd.randrange(1, n + 1)])
+    use_rope, use_norm = rnd.random() < 0.7, rnd.random() < 0.5
+    g = gen(case % 100000)
+    d, dkv = H * hd, Hkv * hd
+    qkv, qkvr = rand_bf16((n, d + 2 * dkv), g, 1.5)
+    pos, _ = rotary.build_positions(n, (0, 0, 0), 0)
+    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48) if hd == 128 else (16, 24, 24))
+    n_seg = rnd.randrange(1, 4) if n >= 3 else 1
+    ends = sorted(rnd.sample(range(1, n), n_seg - 1)) + [n] if n_seg > 1 else [n]
+    qw, kw = 1 + 0.3 * torch.randn(n_seg, hd, generator=g), 1 + 0.3 * torch.randn(n_seg, hd, generator=g)
+    kwargs = dict(causal_prefix=P, n_kv_heads=Hkv)
+    if use_rope:
+        kwargs.update(cos=cos.to(dev()), sin=sin.to(dev()))
+    if use_norm and use_rope:
+        kwargs.update(qk_norm=(qw.to(dev()), kw.to(dev()), ends, 1e-6))
+    variant = rnd.choice([0, 0, 1])
+    prev = ops.set_variant("attn", variant)
+    try:
+        o = ops.attention(qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:], H, hd, **kwargs)
+    finally:
+        ops.set_variant("attn", prev)
+    qn, kn = qkvr[:, :d].view(n, H, hd).clone(), qkvr[:, d:d + dkv].view(n, Hkv, hd).clone()
+    if use_norm and use_rope:
+        s0 = 0
+        for i, e in enumerate(ends):
+            qn[s0:e] = O.rms_norm(qn[s0:e], qw[i], 1e-6)
+            kn[s0:e] = O.rms_norm(kn[s0:e], kw[i], 1e-6)
+            s0 = e
+    if use_rope:
+        qn, kn = O.apply_mrope(qn, cos, sin), O.apply_mrope(kn, cos, sin)
+    want = O.attention(qn, kn, qkvr[:, d + dkv:].view(n, Hkv, hd), kv_end=O.hybrid_kv_end(n, P) if P else None)
+    assert_close(o, want.reshape(n, d), 0.9999, 1e-2,
+                 f"attention sweep n={n} H={H}/{Hkv} hd={hd} P={P} rope={use_rope} norm={use_norm} variant={variant}")
+
+
+@pytest.mark.parametrize("case", _sweep(20251, 20))
+def test_gemm_shape_sweep(case):
+    """Random valid GEMM shapes (ragged M and N, K any multiple of the k-tile pair), every epilogue, both pipelines,
+    bf16 and e4m3, output written into a column window of a wider tensor."""
+    import random
+    rnd = random.Random(case)
+    fp8 = rnd.random() < 0.35
+    M = rnd.choice([rnd.randrange(1, 64), rnd.randrange(64, 600), rnd.randrange(600, 1400)])
+    N = 8 * rnd.randrange(1, 160)
+    K = (256 if fp8 else 128) * rnd.randrange(1, 9)
+    epi = rnd.choice(["none", "swiglu", "gate_residual"])
+    variant = rnd.choice([0, 0, 1])
+    g = gen(case % 100000)
+    a, ar = rand_bf16((M, K), g)
+    w, wr = rand_bf16((N, K), g, 0.05)
+    w2, w2r = rand_bf16((N, K), g, 0.05)
+    r, rr = rand_bf16((M, N), g)
+    gate = torch.randn(N, generator=g)
+    pad = 8 * rnd.randrange(0, 4)
+    wide = torch.zeros((M, N + 2 * pad), dtype=torch.bfloat16, device=dev())
+    out = wide[:, pad:pad + N]
+    prev = ops.set_variant("gemm", variant)
+    try:
+        if fp8:
+            aq, sa = ops.quant_rows(a)
+            wq, sw = ops.quant_rows(w)
+            w2q, sw2 = ops.quant_rows(w2)
+            kw = dict(w2q=w2q, sw2=sw2) if epi == "swiglu" else dict(residual=r, gate=gate.to(dev())) if epi == "gate_residual" else {}
+            ops.gemm_fp8(aq, sa, wq, sw, epilogue=epi, out=out, **kw)
+            lin = O.fp8_linear
+        else:
+            kw = dict(w2=w2) if epi == "swiglu" else dict(residual=r, gate=gate.to(dev())) if epi == "gate_residual" else {}
+            ops.gemm(a, w, epilogue=epi, out=out, **kw)
+            lin = lambda A, W: A @ W.t()
+    finally:
+        ops.set_variant("gemm", prev)
+    if epi == "swiglu":
+        want = torch.nn.functional.silu(lin(ar, wr)) * lin(ar, w2r)
+    elif epi == "gate_residual":
+        want = rr + gate * lin(ar, wr)
+    else:
+        want = lin(ar, wr)
+    assert_close(out, want, 0.9999, 1e-2, f"gemm sweep {M}x{N}x{K} {epi} fp8={fp8} variant={variant} pad={pad}")
+    if pad:
+        assert float(wide[:, :pad].abs().max()) == 0.0 and float(wide[:, pad + N:].abs().max()) == 0.0
