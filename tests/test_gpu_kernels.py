@@ -516,3 +516,50 @@ def test_gemm_shape_sweep(case):
     assert_close(out, want, 0.9999, 1e-2, f"gemm sweep {M}x{N}x{K} {epi} fp8={fp8} variant={variant} pad={pad}")
     if pad:
         assert float(wide[:, :pad].abs().max()) == 0.0 and float(wide[:, pad + N:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("case", _sweep(20252, 8))
+def test_grouped_gemm_sweep(case):
+    """1 to 12 row segments (more than one launch batch holds) of random lengths, with gaps and empty segments, SwiGLU
+    or gated residual, each with its own weights: equal to the per-segment launches bit for bit and within tolerance of
+    the fp32 product."""
+    import random
+    rnd = random.Random(case)
+    n_seg = rnd.randrange(1, 13)
+    K, N = 128 * rnd.randrange(1, 4), 8 * rnd.randrange(4, 60)
+    epi = rnd.choice(["swiglu", "gate_residual"])
+    segs, row = [], rnd.randrange(0, 5)
+    for _ in range(n_seg):
+        ln = rnd.choice([0, rnd.randrange(1, 40), rnd.randrange(40, 400)])
+        segs.append((row, ln))
+        row += ln + rnd.choice([0, 0, rnd.randrange(1, 9)])
+    M = row + rnd.randrange(0, 4)
+    if M == 0:
+        M, segs = 8, [(0, 8)] + segs[1:]
+    g = gen(case % 100000)
+    a, ar = rand_bf16((M, K), g)
+    ws = [rand_bf16((N, K), g, 0.05) for _ in segs]
+    w2s = [rand_bf16((N, K), g, 0.05) for _ in segs]
+    r, rr = rand_bf16((M, N), g)
+    gates = [rnd.choice([None, torch.randn(N, generator=g)]) for _ in segs]
+    gd = [None if x is None else x.to(dev()) for x in gates]
+    if epi == "swiglu":
+        out = torch.zeros((M, N), dtype=torch.bfloat16, device=dev())
+        ops.grouped_gemm(a, [w[0] for w in ws], segs, w2s=[w[0] for w in w2s], epilogue="swiglu", out=out)
+        ref = torch.zeros_like(out)
+        want = torch.zeros(M, N)
+        for i, (s0, ln) in enumerate(segs):
+            if ln:
+                ops.gemm(a[s0:s0 + ln], ws[i][0], w2=w2s[i][0], epilogue="swiglu", out=ref[s0:s0 + ln])
+                want[s0:s0 + ln] = torch.nn.functional.silu(ar[s0:s0 + ln] @ ws[i][1].t()) * (ar[s0:s0 + ln] @ w2s[i][1].t())
+    else:
+        out = r.clone()
+        ops.grouped_gemm(a, [w[0] for w in ws], segs, epilogue="gate_residual", residual=out, gates=gd, out=out)
+        ref = r.clone()
+        want = rr.clone()
+        for i, (s0, ln) in enumerate(segs):
+            if ln:
+                ops.gemm(a[s0:s0 + ln], ws[i][0], epilogue="gate_residual", residual=ref[s0:s0 + ln], gate=gd[i], out=ref[s0:s0 + ln])
+                want[s0:s0 + ln] = rr[s0:s0 + ln] + (1.0 if gates[i] is None else gates[i]) * (ar[s0:s0 + ln] @ ws[i][1].t())
+    assert torch.equal(out, ref), f"grouped != per-segment launches ({n_seg} segments, {epi})"
+    assert_close(out, want, 0.9999, 1e-2, f"grouped sweep {n_seg} segments {M}x{N}x{K} {epi}")
