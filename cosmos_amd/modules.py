@@ -34,6 +34,31 @@ def _as2d(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def _batch_size(t: Optional[torch.Tensor], batched_dim: int) -> int:
+    return t.shape[0] if t is not None and t.dim() == batched_dim else 1
+
+
+def _sample(t: Optional[torch.Tensor], b: int, batched_dim: int, batch: int) -> Optional[torch.Tensor]:
+    """Entry b of a batched argument (kept batched, size 1); an argument of batch size 1 is shared by all samples."""
+    if t is None or t.dim() != batched_dim or t.shape[0] == 1:
+        return t
+    if t.shape[0] != batch:
+        raise ValueError(f"batch size mismatch: {t.shape[0]} vs {batch}")
+    return t[b:b + 1]
+
+
+def _over_batch(fn, batch: int, return_dict: bool):
+    """Run fn(b) for every sample and join the results (tuples or dicts of tensors / None) along the batch axis.  The
+    joint sequence of a forward is ONE sample (attention spans it), so a batch is a loop, e.g. the conditional and the
+    unconditional pass of classifier-free guidance given as a batch of two."""
+    outs = [fn(b) for b in range(batch)]
+    # per-sample results carry a leading batch axis of size 1, except the 2-D joint sequence of the stack's dict form
+    cat = lambda xs: None if xs[0] is None else (torch.cat(xs, 0) if xs[0].dim() >= 3 else torch.stack(xs, 0))
+    if isinstance(outs[0], dict):
+        return {k: cat([o[k] for o in outs]) for k in outs[0]}
+    return tuple(cat([o[i] for o in outs]) for i in range(len(outs[0])))
+
+
 class Workspace:
     """Caller-owned scratch tensors of one (n_tokens, d, hidden) shape, reused by every block."""
 
@@ -438,6 +463,13 @@ class DMStack(nn.Module):
                 encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
                 return_dict: bool = False, context_cache: Optional["ContextCache"] = None):
         c = self.cfg
+        batch = _batch_size(hidden_states, 3)
+        if batch > 1:
+            ts = timestep.reshape(-1)
+            return _over_batch(lambda b: self.forward(hidden_states[b:b + 1], ts[b:b + 1] if ts.numel() == batch else ts,
+                                                      _sample(encoder_hidden_states, b, 3, batch),
+                                                      _sample(action_states, b, 3, batch), return_dict, context_cache),
+                               batch, return_dict)
         if context_cache is not None:
             return self._forward_cached(hidden_states, timestep, action_states, return_dict, context_cache)
         parts = []
@@ -563,6 +595,13 @@ class DMTransformer(nn.Module):
         model width; action_states: [1, n_action, action_dim].  Returns the velocity prediction, latents-shaped and
         bf16 (plus the action prediction when there is an action stream)."""
         c = self.cfg
+        batch = _batch_size(hidden_states, 5)
+        if batch > 1:
+            ts = timestep.reshape(-1)
+            return _over_batch(lambda b: self.forward(hidden_states[b:b + 1], ts[b:b + 1] if ts.numel() == batch else ts,
+                                                      _sample(encoder_hidden_states, b, 3, batch),
+                                                      _sample(action_states, b, 3, batch), return_dict),
+                               batch, return_dict)
         dt = self.proj_in.weight.dtype
         tok = self.proj_in(self.patchify(hidden_states[0].to(dt)))
         act = None

@@ -493,3 +493,28 @@ def test_full_size_block_sampled_rows(name):
         assert_close(got, want, BF16_COS, BF16_REL, f"{name} full-size block, sampled rows")
         assert float((want - upd).abs().max()) > 0.5
         assert_close(got.float().cpu() - upd, want - upd, 0.999, BF16_REL, f"{name} full-size block update")
+
+
+def test_batched_forward_is_a_loop_over_samples():
+    """A batch (e.g. the conditional and unconditional pass of classifier-free guidance as a batch of two) gives the
+    per-sample results, sample by sample: per-sample timesteps and contexts, a shared context when its batch is 1."""
+    from cosmos_amd import DMTransformer
+    cfg = DMConfig("bt", 256, 2, 128, 512, 2, (2, 3, 4), n_text=12, n_action=5, n_branches=3, qk_norm=True)
+    m = DMTransformer(cfg, latent_channels=4, action_dim=6, device=dev())
+    m.reset_parameters(5)
+    g = torch.Generator(device=dev()).manual_seed(5)
+    lat = torch.randn((2, 4, 2, 6, 8), generator=g, device=dev())
+    ctx = torch.randn((2, 12, 256), generator=g, device=dev()).to(torch.bfloat16)
+    act = torch.randn((2, 5, 6), generator=g, device=dev())
+    t = torch.tensor([100.0, 900.0], device=dev())
+    both = m(lat, t, encoder_hidden_states=ctx, action_states=act)
+    assert both[0].shape == (2, 4, 2, 6, 8) and both[1].shape[0] == 2
+    for b in range(2):
+        one = m(lat[b:b + 1], t[b:b + 1], encoder_hidden_states=ctx[b:b + 1], action_states=act[b:b + 1])
+        assert torch.equal(both[0][b:b + 1], one[0]) and torch.equal(both[1][b:b + 1], one[1])
+    assert not torch.equal(both[0][0], both[0][1])
+    shared = m(lat, t, encoder_hidden_states=ctx[:1], action_states=act)          # one context for both samples
+    assert torch.equal(shared[0][0], both[0][0]) and not torch.equal(shared[0][1], both[0][1])
+    d = m.stack(torch.randn((2, cfg.n_video, 256), generator=g, device=dev()).to(torch.bfloat16), t, encoder_hidden_states=ctx,
+                action_states=torch.randn((2, 5, 256), generator=g, device=dev()).to(torch.bfloat16), return_dict=True)
+    assert d["sample"].shape == (2, cfg.n_video, 256) and d["joint"].shape == (2, cfg.n_tokens, 256)
