@@ -49,3 +49,44 @@ def test_stack_segments_meta():
     assert st.segments() == [(0, 3, 0, False), (3, 8, 1, True), (11, 2, 2, True)]
     cfg1 = DMConfig("t", 128, 2, 64, 256, 0, (2, 2, 2), n_text=3, mrope_sections=(16, 24, 24))
     assert DMStack(cfg1, device="meta").segments() == [(0, 3, 0, False), (3, 8, 0, True)]
+
+
+@pytest.mark.parametrize("order,corrector,solver_type,grid", [(1, True, "bh2", "plain"), (2, True, "bh2", "plain"), (3, True, "bh1", "library"),
+                                                              (2, False, "bh2", "library"), (3, True, "bh2", "plain")])
+def test_unipc_coefficient_rows_on_the_host(monkeypatch, order, corrector, solver_type, grid):
+    """The stepper's host side (folding corrector + predictor + data prediction into three coefficient rows, history
+    and buffer rotation) with the fused launch replaced by the same linear combinations in float64 on the CPU:
+    must reproduce the tensor-level oracle sampler step by step."""
+    import numpy as np
+    from cosmos_amd import ops, sampler
+    from oracle import unipc as U
+
+    def fake_multistep(x, v_cond, v_uncond, guidance, coef, hist, outs):
+        v = v_cond.double() if v_uncond is None else v_uncond.double() + guidance * (v_cond.double() - v_uncond.double())
+        ins = [x.double().clone(), v] + [h.double().clone() for h in hist]       # read everything before any write
+        for row, out in zip(coef, outs):
+            out.copy_(sum(c * t for c, t in zip(row, ins)))
+
+    monkeypatch.setattr(ops, "cfg_multistep", fake_multistep)
+    steps, n, guidance = 7, 64, 2.5
+    sig = U.flow_sigmas(steps, 3.0) if grid == "plain" else U.diffusers_flow_sigmas(steps, 3.0)
+    st = sampler.UniPCStepper(sig, guidance_scale=guidance, solver_order=order, solver_type=solver_type,
+                              use_corrector=corrector)
+    ref = U.UniPCSampler(sig, solver_order=order, solver_type=solver_type, use_corrector=corrector)
+    g = torch.Generator().manual_seed(order)
+    x = torch.randn(n, generator=g, dtype=torch.float64)
+    xr = x.numpy().copy()
+    for i in range(steps):
+        vc = torch.randn(n, generator=g, dtype=torch.float64)
+        vu = torch.randn(n, generator=g, dtype=torch.float64)
+        x = st.step(vc, vu, x)
+        xr = ref.step((vu + guidance * (vc - vu)).numpy(), xr)
+        assert st.this_order == ref.this_order
+        assert np.allclose(x.numpy(), xr, rtol=1e-9, atol=1e-9), f"step {i}"
+    assert len(st.m_hist) <= order and len(st._spare) <= 1
+    with pytest.raises(RuntimeError):
+        st.step(vc, vu, x)
+    with pytest.raises(ValueError):
+        sampler.UniPCStepper([0.5, 0.7, 0.0])
+    with pytest.raises(ValueError):
+        sampler.UniPCStepper(sig, solver_order=4)
