@@ -30,6 +30,7 @@ class QkNorm(C.Structure):
 SIGNATURES = {
     "cdm_version": (_I32, []),
     "cdm_last_error": (C.c_char_p, []),
+    "cdm_source_hash": (C.c_char_p, []),
     "cdm_device_count": (_I32, []),
     "cdm_set_variant": (_I32, [C.c_char_p, _I32]),
     "cdm_adaln_rmsnorm_bf16": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
@@ -61,14 +62,21 @@ def lib_path() -> str:
 
 
 def load():
-    """Return the loaded library (building it first only if no built library exists)."""
+    """Return the loaded library.  The in-tree build is (re)built first if it is missing or was built from other
+    sources than the ones present (a stale build is never run); a library named by COSMOS_DM_LIB is taken as is."""
     global _LIB
     with _LOCK:
         if _LIB is not None:
             return _LIB
         path = lib_path()
-        if not os.path.exists(path):
-            _build.build(verbose=False)
+        if path == _build.LIB_PATH:
+            want = _build.source_hash()
+            if _build.built_hash(path) != want:
+                _build.build(verbose=False)
+                if _build.built_hash(path) != want:
+                    raise RuntimeError(f"{path} does not carry the hash of the present sources after a rebuild")
+        elif not os.path.exists(path):
+            raise RuntimeError(f"COSMOS_DM_LIB={path} does not exist")
         lib = C.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)     # AttributeError here = the library does not export the ABI

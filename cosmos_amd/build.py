@@ -1,6 +1,7 @@
 """Builds libcosmos_dm_hip.so (gfx950) in-tree with hipcc.  ``python -m cosmos_amd.build``."""
 from __future__ import annotations
 
+import hashlib
 import os
 import shutil
 import subprocess
@@ -18,6 +19,33 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+HASH_MARKER = b"CDM_SRC_HASH="
+
+
+def source_hash() -> str:
+    """16 hex digits over every file the library is built from (kernels, shared headers, the public header)."""
+    h = hashlib.sha256()
+    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".h"))]
+    files += [os.path.join(INCLUDE, f) for f in sorted(os.listdir(INCLUDE)) if f.endswith(".h")]
+    for path in files:
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def built_hash(path: str = LIB_PATH) -> str:
+    """The source hash a built library carries ("" if the file is missing or carries none)."""
+    try:
+        with open(path, "rb") as fh:
+            blob = fh.read()
+    except OSError:
+        return ""
+    i = blob.find(HASH_MARKER)
+    return blob[i + len(HASH_MARKER):i + len(HASH_MARKER) + 16].decode("ascii", "replace") if i >= 0 else ""
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -27,7 +55,7 @@ def _hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *FLAGS, f'-DCDM_SOURCE_HASH="{source_hash()}"', "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr[-4000:]}")

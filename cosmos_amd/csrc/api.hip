@@ -37,7 +37,15 @@ int32_t cdm_require_device(void) {
 
 int32_t cdm_get_variant(int which) { return g_variant[which].load(std::memory_order_relaxed); }
 
-extern "C" int32_t cdm_version(void) { return 100; }
+#ifndef CDM_SOURCE_HASH
+#define CDM_SOURCE_HASH "unknown"
+#endif
+// the marker lets a loader read the hash from the file without loading it
+static const char kSourceHash[] = "CDM_SRC_HASH=" CDM_SOURCE_HASH;
+
+extern "C" int32_t cdm_version(void) { return 101; }
+
+extern "C" const char* cdm_source_hash(void) { return kSourceHash + 13; }
 
 extern "C" const char* cdm_last_error(void) { return g_err; }
 

@@ -78,8 +78,10 @@ class _Update:
         h = _lam(st) - lam_s0
         hh = -h
         h_phi_1 = math.expm1(hh)
-        B_h = h_phi_1 if solver_type == "bh2" else hh
         finite = math.isfinite(hh)
+        # B(h) = h ("bh1") has no limit when the step starts at sigma = 1 (lambda = -inf, h infinite), while
+        # e^h - 1 ("bh2") tends to -1; both variants agree to first order in h, so that step takes the bh2 form
+        B_h = h_phi_1 if (solver_type == "bh2" or not finite) else hh
         # divided-difference abscissae of the older predictions (an abscissa at -inf switches its term off)
         rks = [(_lam(sg) - lam_s0) / h if finite else 0.0 for sg in older] + [1.0]
         inv_rk = [0.0 if (rk == 0.0 or math.isinf(rk)) else 1.0 / rk for rk in rks[:-1]]

@@ -50,6 +50,10 @@ typedef enum cdm_epilogue {
 /* Library version (major*10000 + minor*100 + patch). */
 int32_t cdm_version(void);
 
+/* Hash of the sources this library was built from (16 hex digits): a loader compares it with the hash of the
+ * sources it sees and refuses, or rebuilds, a stale build. */
+const char* cdm_source_hash(void);
+
 /* Message for the last non-zero status returned on this thread ("" if none). */
 const char* cdm_last_error(void);
 

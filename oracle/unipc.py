@@ -77,7 +77,8 @@ def unip_update(x, m_hist: Sequence, sig_hist: Sequence[float], sigma_t: float, 
     h = lam_t - lam_s0
     hh = -h
     h_phi_1 = math.expm1(hh)
-    B_h = math.expm1(hh) if solver_type == "bh2" else hh
+    # a step that starts at sigma = 1 has infinite h: B(h) = h ("bh1") has no limit there, e^h - 1 ("bh2") tends to -1
+    B_h = math.expm1(hh) if (solver_type == "bh2" or not math.isfinite(hh)) else hh
     rks, D1s = [], []
     for i in range(1, order):
         rk = (_lam(sig_hist[-1 - i]) - lam_s0) / h
@@ -105,7 +106,8 @@ def unic_update(x_last, m_hist: Sequence, sig_hist: Sequence[float], m_t, sigma_
     h = lam_t - lam_s0
     hh = -h
     h_phi_1 = math.expm1(hh)
-    B_h = math.expm1(hh) if solver_type == "bh2" else hh
+    # a step that starts at sigma = 1 has infinite h: B(h) = h ("bh1") has no limit there, e^h - 1 ("bh2") tends to -1
+    B_h = math.expm1(hh) if (solver_type == "bh2" or not math.isfinite(hh)) else hh
     rks, D1s = [], []
     for i in range(1, order):
         rk = (_lam(sig_hist[-1 - i]) - lam_s0) / h

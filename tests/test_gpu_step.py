@@ -86,7 +86,8 @@ def test_cfg_multistep_rows_and_aliasing(n_out, n_hist):
 
 @pytest.mark.parametrize("order,corrector,solver_type,shift,grid", [
     (1, False, "bh2", 1.0, "plain"), (2, True, "bh2", 3.0, "plain"), (3, True, "bh2", 3.0, "plain"),
-    (2, True, "bh1", 5.0, "library"), (3, True, "bh2", 1.0, "library"), (2, False, "bh2", 3.0, "library")])
+    (2, True, "bh1", 5.0, "library"), (3, True, "bh2", 1.0, "library"), (2, False, "bh2", 3.0, "library"),
+    (2, True, "bh1", 3.0, "plain"), (3, True, "bh1", 10.0, "plain")])
 def test_unipc_stepper_matches_oracle(order, corrector, solver_type, shift, grid):
     """The stepper's folded coefficient rows + one fused launch per step against the tensor-level float64 sampler,
     fed with the same random 'model outputs' (so any slip in the algebra shows at once)."""
@@ -106,6 +107,7 @@ def test_unipc_stepper_matches_oracle(order, corrector, solver_type, shift, grid
         v = (vur + guidance * (vcr - vur)).double().numpy()
         xr = ref.step(v, xr)
         assert st.this_order == ref.this_order
+        assert bool(torch.isfinite(x).all()), f"step {i}: non-finite latents"
         err = float((x.double().cpu() - torch.from_numpy(xr)).abs().max())
         assert err < 2e-4 * max(1.0, float(abs(xr).max())), f"step {i}: {err}"
     with pytest.raises(RuntimeError):

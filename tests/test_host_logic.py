@@ -52,7 +52,8 @@ def test_stack_segments_meta():
 
 
 @pytest.mark.parametrize("order,corrector,solver_type,grid", [(1, True, "bh2", "plain"), (2, True, "bh2", "plain"), (3, True, "bh1", "library"),
-                                                              (2, False, "bh2", "library"), (3, True, "bh2", "plain")])
+                                                              (2, False, "bh2", "library"), (3, True, "bh2", "plain"),
+                                                              (1, True, "bh1", "plain"), (2, True, "bh1", "plain"), (3, True, "bh1", "plain")])
 def test_unipc_coefficient_rows_on_the_host(monkeypatch, order, corrector, solver_type, grid):
     """The stepper's host side (folding corrector + predictor + data prediction into three coefficient rows, history
     and buffer rotation) with the fused launch replaced by the same linear combinations in float64 on the CPU:
@@ -82,6 +83,7 @@ def test_unipc_coefficient_rows_on_the_host(monkeypatch, order, corrector, solve
         x = st.step(vc, vu, x)
         xr = ref.step((vu + guidance * (vc - vu)).numpy(), xr)
         assert st.this_order == ref.this_order
+        assert np.isfinite(xr).all() and bool(torch.isfinite(x).all()), f"step {i}: non-finite latents"
         assert np.allclose(x.numpy(), xr, rtol=1e-9, atol=1e-9), f"step {i}"
     assert len(st.m_hist) <= order and len(st._spare) <= 1
     with pytest.raises(RuntimeError):

@@ -147,6 +147,10 @@ def test_full_schedule_is_finite_and_beats_euler(shift, grid):
     e3 = run(grid(80, shift), v, sol, z, solver_order=3)
     assert all(np.isfinite(e) for e in (e1, e2, e3))
     assert e2 < e1 / 8 and e3 < e1 / 8
+    # B(h) = h: a grid that starts at sigma = 1 has an infinite first step, which takes the e^h - 1 form
+    for order in (1, 2, 3):
+        eb = run(grid(80, shift), v, sol, z, solver_order=order, solver_type="bh1")
+        assert np.isfinite(eb) and eb < e1 / 2, (order, eb, e1)
 
 
 def test_diffusers_style_grid_shape():
