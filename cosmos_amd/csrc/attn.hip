@@ -13,6 +13,8 @@
 // the 8 consecutive keys the second product expects.
 // Rotate-half mRoPE (and the QK-RMSNorm ahead of it) is applied in registers: to K while it is re-tiled for the
 // kernel, to Q when the kernel loads its Q fragments (both members of a rotary pair sit in the same lane).
+#include <mutex>
+
 #include "cdm_common.h"
 
 namespace {
@@ -759,4 +761,62 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
         return rc;
     return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, n_kv_heads, head_dim, qk_norm,
                                     nullptr, 0, causal_prefix, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same operator for callers that can neither allocate nor bring a workspace: the K / V tile images go into a
+// file-scope device array.  In host code the array's NAME is only a handle; its device address is looked up once
+// per device (hipGetSymbolAddress, with that device current) and every use below goes through that pointer.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int64_t kStaticScratchBytes = CDM_ATTN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};      // device address of `scratch` on each device (null = not looked up yet)
+
+// address of the current device's copy of `scratch`
+int32_t static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        CDM_FAIL(CDM_ERR_NO_DEVICE, "attn_fwd_static: no current device (%s)", hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            CDM_FAIL(CDM_ERR_LAUNCH, "attn_fwd_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                     hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return CDM_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t cdm_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int32_t cdm_attn_fwd_static_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
+                                            int64_t ldv, const float* cos, const float* sin, void* o, int64_t ldo,
+                                            int64_t n_tokens, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
+                                            const cdm_qk_norm* qk_norm, int64_t causal_prefix, void* stream) {
+    CDM_REQUIRE(n_tokens >= 0 && n_kv_heads > 0 && head_dim > 0, CDM_ERR_BAD_ARG, "attn_fwd_static: bad sizes");
+    CDM_REQUIRE(n_tokens <= 65535ll * BN, CDM_ERR_BAD_SHAPE, "attn_fwd_static: sizes out of range");
+    const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim);
+    CDM_REQUIRE(need <= kStaticScratchBytes, CDM_ERR_BAD_SHAPE,
+                "attn_fwd_static: K/V tile images of %lld tokens x %d K/V heads x %d need %lld bytes, the built-in "
+                "scratch holds %lld; use cdm_attn_fwd_bf16 with a caller-owned workspace",
+                (long long)n_tokens, n_kv_heads, head_dim, (long long)need, (long long)kStaticScratchBytes);
+    void* ws = nullptr;
+    if (n_tokens > 0) {
+        int32_t rc = cdm_require_device();
+        if (rc) return rc;
+        if ((rc = static_scratch(&ws))) return rc;
+    }
+    return cdm_attn_fwd_bf16(q, ldq, k, ldk, v, ldv, cos, sin, o, ldo, n_tokens, n_heads, n_kv_heads, head_dim, ws,
+                             kStaticScratchBytes, qk_norm, causal_prefix, stream);
 }

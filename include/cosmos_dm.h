@@ -199,6 +199,23 @@ int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, c
                                  void* stream);
 
 /*
+ * cdm_attn_fwd_bf16 for callers that cannot allocate device memory or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference; the
+ * operator and all other arguments are those of cdm_attn_fwd_bf16.  The K / V tile images go into a device array
+ * built into the library (CDM_ATTN_STATIC_SCRATCH_BYTES per GPU, held until the process ends); the call allocates
+ * nothing.  Shapes whose images (cdm_attn_workspace_bytes) exceed that size are rejected with CDM_ERR_BAD_SHAPE.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream are ordered and need no clearing in between (every call rewrites all
+ * tiles it reads, padding included).
+ */
+#define CDM_ATTN_STATIC_SCRATCH_BYTES (32ll << 20)
+int64_t cdm_attn_static_scratch_bytes(void);
+int32_t cdm_attn_fwd_static_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
+                                 const float* cos, const float* sin, void* o, int64_t ldo, int64_t n_tokens,
+                                 int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
+                                 int64_t causal_prefix, void* stream);
+
+/*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each
  * (README.md:53,74 - per-modality weights around one shared attention).  Equivalent to
  * cdm_gemm_bf16 on rows [seg_start[g], seg_start[g] + seg_len[g]) with W[g] (and W2[g], gate[g]).

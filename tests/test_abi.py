@@ -50,6 +50,12 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 1, 48, fake, 1 << 20, None, 0, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 16, 1, 1, 64, fake, 16, None, 0, None) == _lib.ERR_BAD_ARG
     assert "workspace" in _lib.last_error()
+    # the entry point that allocates nothing rejects shapes whose tile images exceed its built-in scratch
+    assert lib.cdm_attn_static_scratch_bytes() == 32 << 20
+    assert lib.cdm_attn_fwd_static_bf16(fake, 4096, fake, 4096, fake, 4096, None, None, fake, 4096, 56320, 32, 32, 128, None, 0,
+                                        None) == _lib.ERR_BAD_SHAPE
+    assert "scratch" in _lib.last_error()
+    assert lib.cdm_attn_fwd_static_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 0, 1, 1, 64, None, 0, None) == _lib.OK
     assert lib.cdm_mrope_qk_bf16(fake, 64, None, 0, fake, fake, 4, 1, 32, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_quant_rows_e4m3(fake, 128, fake, fake, 4, 100, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_set_variant(b"nope", 0) == _lib.ERR_BAD_ARG
