@@ -113,6 +113,8 @@ def main():
     ap.add_argument("--attn-variant", type=int, default=0)
     ap.add_argument("--gemm-variant", type=int, default=0)
     ap.add_argument("--rope", default="in_attention", choices=["in_attention", "gemm_epilogue", "streaming"])
+    ap.add_argument("--residual", default="fp32", choices=["fp32", "bf16"],
+                    help="dtype the residual stream is kept in between blocks (fp32 = the default of a stack)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
@@ -135,6 +137,7 @@ def main():
     cfg = CONFIGS[args.workload]
     if args.blocks:
         cfg = dataclasses.replace(cfg, n_blocks=args.blocks)
+    cfg = dataclasses.replace(cfg, residual_fp32=(args.residual == "fp32"))
     _lib.load()
     if args.workload == "C1" and args.steps == 3:
         args.steps = 10
@@ -200,7 +203,8 @@ def main():
         tf = cfg.gemm_flops_per_block() / (per_block["gemm"] * 1e-3) / 1e12
         kernels["gemm"] = {"ms_per_block": round(per_block["gemm"], 3), "tflops": round(tf, 1), "frac_of_mfma_peak": round(tf / gemm_peak, 4)}
     nd = cfg.n_tokens * cfg.d_model
-    hbm_bytes = {"norm": 2 * (3 if cfg.fp8 else 4) * nd,       # two norms per block: read bf16, write bf16 (or e4m3)
+    xb = 4 if cfg.residual_fp32 else 2                         # bytes per element of the residual stream
+    hbm_bytes = {"norm": 2 * (xb + (1 if cfg.fp8 else 2)) * nd,  # two norms per block: read the stream, write bf16 (or e4m3)
                  "pack_kv": 8 * nd + 8 * cfg.n_tokens * (cfg.head_dim // 2),   # K, V in; two tile images out; cos/sin
                  "quant": 2 * 3 * nd + 3 * cfg.n_tokens * cfg.hidden,           # attention output and SwiGLU hidden -> e4m3
                  "rope": 8 * nd}
@@ -216,7 +220,8 @@ def main():
         "config": {"workload": f"{cfg.name}: {cfg.n_blocks} DM blocks, d={cfg.d_model}, {cfg.n_heads}x{cfg.head_dim} heads, "
                                f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
-                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope},
+                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope,
+                   "residual_stream": args.residual},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4),
                      "traffic": ATTN_TRAFFIC_BYTES.get((cfg.n_tokens, cfg.n_heads, cfg.head_dim))

@@ -16,7 +16,7 @@ _LIB = None
 
 OK = 0
 ERR_BAD_ARG, ERR_BAD_SHAPE, ERR_BAD_ALIGN, ERR_NO_DEVICE, ERR_LAUNCH, ERR_UNSUPPORTED = -1, -2, -3, -4, -5, -6
-EPI_NONE, EPI_SWIGLU, EPI_GATE_RESIDUAL, EPI_ROPE_QK = 0, 1, 2, 3
+EPI_NONE, EPI_SWIGLU, EPI_GATE_RESIDUAL, EPI_ROPE_QK, EPI_GATE_RESIDUAL_F32 = 0, 1, 2, 3, 4
 
 _P, _I64, _I32, _F32 = C.c_void_p, C.c_int64, C.c_int32, C.c_float
 
@@ -35,6 +35,8 @@ SIGNATURES = {
     "cdm_set_variant": (_I32, [C.c_char_p, _I32]),
     "cdm_adaln_rmsnorm_bf16": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
     "cdm_adaln_rmsnorm_quant_e4m3": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
+    "cdm_adaln_rmsnorm_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
+    "cdm_adaln_rmsnorm_f32_quant_e4m3": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
     "cdm_quant_rows_e4m3": (_I32, [_P, _I64, _P, _P, _I64, _I64, _P]),
     "cdm_gemm_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P, _P, _P, _I64,
                              _I32, _P]),

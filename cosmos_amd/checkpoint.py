@@ -6,7 +6,7 @@ keys the Reasoner-only model drops, and conversion_mapping.py:920-941, the renam
     ``add_q_proj, add_k_proj, add_v_proj, to_add_out, norm_added_q, norm_added_k``;
   * the DM branch's norms and MLP carry ``moe_gen`` in their names;
   * top level: ``proj_in., proj_out., time_embedder.``, ``action_proj_in., action_proj_out., action_modality_embed``,
-    ``audio_*`` (sound tower, not handled here).
+    ``audio_proj_in., audio_proj_out., audio_modality_embed`` (the sound stream).
 Only the substring ``moe_gen`` is attested for the DM norms / MLP; the patterns below accept it anywhere in the
 module name together with the usual ``gate_proj / up_proj / down_proj / input_layernorm / post_attention_layernorm``
 words.  The AR twin's norms and MLP use the plain Qwen3-VL names (``input_layernorm``, ``post_attention_layernorm``,
@@ -51,8 +51,15 @@ _RULES: List[Tuple[str, Tuple, Optional[int]]] = [
     (_LAYER + r"[\w.]*ada(?:LN|ln)[\w.]*\.(weight|bias)$", ("adaln", None), None),
 ]
 _TOP = [r"^proj_in\.", r"^proj_out\.", r"^time_embedder\.", r"^action_proj_in\.", r"^action_proj_out\.",
-        r"^action_modality_embed$", r"^norm_out\."]
+        r"^action_modality_embed$", r"^audio_proj_in\.", r"^audio_proj_out\.", r"^audio_modality_embed$", r"^norm_out\."]
 _COMPILED = [(re.compile(rx), tgt, br) for rx, tgt, br in _RULES]
+
+
+def _copy_exact(dst: torch.Tensor, t: torch.Tensor) -> None:
+    """copy_ broadcasts silently; a checkpoint tensor must have exactly the shape of its destination."""
+    if tuple(dst.shape) != tuple(t.shape):
+        raise RuntimeError(f"shape {tuple(t.shape)} does not match the model's {tuple(dst.shape)}")
+    dst.copy_(t)
 
 
 def classify(key: str):
@@ -99,6 +106,9 @@ def load_generator_weights(model, source: Union[str, Iterable[str], Mapping[str,
         layer, tgt, br = c
         try:
             if tgt[0] == "top":
+                if hasattr(model, "top_level_keys") and key not in model.top_level_keys():
+                    unexpected.append(key)          # an edge this model was built without (e.g. no audio stream)
+                    continue
                 _assign_top(model, key, t)
                 seen.add(key)
             else:
@@ -110,22 +120,22 @@ def load_generator_weights(model, source: Union[str, Iterable[str], Mapping[str,
                     # rows of the fused weight: [q: d | k: d_kv | v: d_kv] (d_kv < d under grouped-query attention)
                     dkv = blk.attn.n_kv_heads * blk.attn.head_dim
                     r0 = (0, d, d + dkv)[tgt[1]]
-                    blk.attn.qkv_weight[br].data[r0:r0 + (d if tgt[1] == 0 else dkv)].copy_(t)
+                    _copy_exact(blk.attn.qkv_weight[br].data[r0:r0 + (d if tgt[1] == 0 else dkv)], t)
                     seen.add(f"layers.{layer}.qkv.{br}.{tgt[1]}")
                 elif tgt[0] == "attn":
-                    getattr(blk.attn, tgt[1])[br].data.copy_(t)
+                    _copy_exact(getattr(blk.attn, tgt[1])[br].data, t)
                     seen.add(f"layers.{layer}.{tgt[1]}.{br}")
                 elif tgt[0] == "qknorm":
                     if not blk.attn.qk_norm:
                         unexpected.append(key)
                         continue
-                    getattr(blk.attn, tgt[1]).data[br].copy_(t)
+                    _copy_exact(getattr(blk.attn, tgt[1]).data[br], t)
                     seen.add(f"layers.{layer}.{tgt[1]}.{br}")
                 elif tgt[0] == "block":
-                    getattr(blk, tgt[1])[br].data.copy_(t)
+                    _copy_exact(getattr(blk, tgt[1])[br].data, t)
                     seen.add(f"layers.{layer}.{tgt[1]}.{br}")
                 else:   # adaLN projection of the block
-                    getattr(blk.adaLN_modulation, tgt[-1]).data.copy_(t)
+                    _copy_exact(getattr(blk.adaLN_modulation, tgt[-1]).data, t)
                     seen.add(f"layers.{layer}.adaLN.{tgt[-1]}")
             loaded.append(key)
         except (RuntimeError, AttributeError) as e:      # shape mismatch or a part this model does not have

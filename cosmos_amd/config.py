@@ -15,8 +15,9 @@ class DMConfig:
     n_blocks: int
     grid: Tuple[int, int, int]               # video latent grid T x H x W
     n_text: int = 0                          # text tokens placed before the video tokens
-    n_action: int = 0                        # action tokens placed after the video tokens
-    n_branches: int = 1                      # weight sets (1 = shared, 3 = text / video / action)
+    n_action: int = 0                        # action tokens placed at the end of the joint sequence
+    n_audio: int = 0                         # audio (sound) tokens placed after the video tokens, before the action tokens
+    n_branches: int = 1                      # weight sets (1 = shared, 2 = text / generator, 3 = + action, 4 = + audio)
     mrope_sections: Tuple[int, int, int] = (32, 48, 48)   # channels per axis (t, h, w), sum = head_dim
     rope_base: float = 10000.0
     rope_layout: str = "chunked"
@@ -25,6 +26,7 @@ class DMConfig:
     qk_norm: bool = False                    # per-head RMSNorm of Q and K ahead of the rotation
     hybrid_mask: bool = False                # text run causal and blind to the generator tokens (else full attention)
     n_kv_heads: Optional[int] = None         # K / V heads (None = n_heads; fewer = grouped-query attention)
+    residual_fp32: bool = True               # residual stream of a stack kept in fp32 between blocks (else bf16)
     seed: int = 1234
 
     @property
@@ -37,7 +39,7 @@ class DMConfig:
 
     @property
     def n_tokens(self) -> int:
-        return self.n_text + self.n_video + self.n_action
+        return self.n_text + self.n_video + self.n_audio + self.n_action
 
     def gemm_flops_per_block(self) -> float:
         n, d, h = self.n_tokens, self.d_model, self.hidden

@@ -113,15 +113,20 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-template <int HD, int QS, class Mid>
+// NEED_MAX = false: the caller has shown that no score of this wave's rows can exceed the reference by more than
+//   2^kSafeLog2 (norm bound |q| max|k|), so the per-tile row maximum and the reference update are dropped altogether.
+template <int HD, int QS, bool NEED_MAX, class Mid>
 __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
                                           f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
                                           bool next_masked, const int (&next_keys_valid)[QS]) {
     constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
-    // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot and
-    // their result is never used - cheaper than a second copy of the step.)
+    // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot, a second
+    // copy of the last tile, and their result is never used - cheaper than a second copy of the step.  When the last
+    // tile is ragged that step masks all of its scores like the one before it masked the padding: the zero keys of the
+    // padding would otherwise show up as scores of -m_ref, and with every real logit far below zero the tail would
+    // move the reference up to them and scale O and l towards zero.)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
@@ -147,8 +152,10 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
                 bf16x2 pp;
-                pp[0] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e]);
-                pp[1] = (__bf16)__builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1]);
+                const float e0 = __builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e]);
+                const float e1 = __builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1]);
+                pp[0] = (__bf16)e0;
+                pp[1] = (__bf16)e1;
                 psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
                 p8[e] = pp[0];
                 p8[e + 1] = pp[1];
@@ -193,17 +200,20 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
         if (i + VWIN < NV) vw[i % VWIN] = v_frag<HD>(sv_cur, (i + VWIN) / TS, (i + VWIN) % TS, lane);
     }
     float mx[QS];
+    if constexpr (NEED_MAX) {
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
+        for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
+    }
     preload_k<HD>(sk_next2, kw, lane);
 #pragma unroll
     for (int i = 0; i < NV * QS; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        if constexpr (NEED_MAX) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(0);
+    if constexpr (!NEED_MAX) return;
 
     // ---- tail.  mx is relative to the reference (the scores are); moving the reference by d means: O and l
     // shrink by 2^-d, the scores already computed for tile j+1 drop by d, and so does the accumulator seed.
@@ -246,8 +256,10 @@ struct PackedParams {
     const bf16_t* q; int64_t ldq;
     const char* kp;              // [n_kv_heads][n_tiles][tile bytes]
     const char* vp;
+    const float* kmax;           // [n_kv_heads][n_tiles]: largest key norm of each tile (after QK-norm / rotation)
     const char* kp_prefix;       // optional tile images of keys that precede those of kp / vp (whole tiles)
     const char* vp_prefix;
+    const float* kmax_prefix;
     int n_prefix_tiles;
     int causal_prefix;           // query rows < causal_prefix see keys <= their own index only; the others see all keys
     bf16_t* o; int64_t ldo;
@@ -261,7 +273,10 @@ struct PackedParams {
 // QS = query sub-tiles (of 32 rows) per wave: QS = 1 -> 8 waves, two per SIMD, 256 registers each;
 // QS = 2 -> 4 waves, one per SIMD with the 512-register budget; every K / V^T fragment read from LDS then feeds
 // two MFMAs instead of one.
-template <int HD, int QS>
+constexpr float kSafeLog2 = 60.0f;      // largest excess over the reference that needs no reference update
+
+// BOUND: take the norm bound of the scores (below) and run the loop without row maxima where it allows
+template <int HD, int QS, bool BOUND>
 __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS, 2 / QS))) void attn_fwd_pipe_kernel(
     const PackedParams p) {
     constexpr int NW = 8 / QS;
@@ -296,6 +311,18 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // ---- Q fragments: rotate-half mRoPE (if tables are given) and the factor log2(e)/sqrt(HD), both in fp32 and
     // with ONE rounding to bf16.  The lane holds channels 16ks + 8kh .. +7 of its query row for every ks, so
     // the partner of a channel in k-step ks (< KS/2) is the same register element of k-step ks + KS/2.
+    // An upper bound of every score of a row: |q| max_k |k| (Cauchy-Schwarz on the very bf16 values the
+    // matrix cores multiply).  kmax_all = the largest key norm of this K/V head over all tiles, prefix included.
+    float kmax_all = 0.0f;
+    if constexpr (BOUND) {
+        const int nm = (p.n_tokens + BN - 1) / BN;
+        const float* km = p.kmax + (int64_t)kv_head * nm;
+        for (int i = lane; i < nm; i += 64) kmax_all = fmaxf(kmax_all, km[i]);
+        const float* kmp = p.kmax_prefix + (int64_t)kv_head * p.n_prefix_tiles;
+        for (int i = lane; i < p.n_prefix_tiles; i += 64) kmax_all = fmaxf(kmax_all, kmp[i]);
+        kmax_all = wave_max(kmax_all);
+    }
+    float qnorm[QS];
     bf16x8 qf[QS][HD / 16];
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
@@ -354,6 +381,19 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             }
             qf[qs][ks] = __builtin_bit_cast(bf16x8, make_uint4(o1[0], o1[1], o1[2], o1[3]));
             qf[qs][ks + KS / 2] = __builtin_bit_cast(bf16x8, make_uint4(o2[0], o2[1], o2[2], o2[3]));
+        }
+        qnorm[qs] = 0.0f;
+        if constexpr (BOUND) {      // norm of the scaled, rotated, rounded query row (the lane and lane ^ 32 hold half each)
+            float ss = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint4 u = __builtin_bit_cast(uint4, qf[qs][ks]);
+                const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { const float a = bf16lo(w[j]), b = bf16hi(w[j]); ss += a * a + b * b; }
+            }
+            ss += __shfl_xor(ss, 32, 64);
+            qnorm[qs] = sqrtf(ss);
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // Q is in registers: from here on vmcnt counts tile loads only
@@ -417,6 +457,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(3 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
     f32x16 s_a[QS][2], s_b[QS][2];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
+    bool need_max = !BOUND;
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
 #pragma unroll
@@ -424,6 +465,10 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         scores_tile<HD>(sk, qf[qs], s_a[qs], lane);
         if (causal_wg || (NT == 1 && ragged)) mask_scores(s_a[qs], klim[qs], lane);
         const float m0 = tile_row_max(s_a[qs]);      // exact first reference: every row has at least one finite score
+        // can any score of this wave's rows exceed its reference by more than 2^kSafeLog2?  (1 % slack for the fp32
+        // accumulation of the dot products and of the norms; a NaN compares as "yes")
+        if constexpr (BOUND)
+            need_max = need_max || __builtin_amdgcn_ballot_w64(!(qnorm[qs] * kmax_all * 1.01f - m0 <= kSafeLog2)) != 0;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             s_a[qs][0][v] -= m0;
@@ -448,7 +493,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // before barrier j: both tiles are complete at barrier j - 1 (neither is the most recently issued group there),
     // and their slots are not refilled before barrier j + 1.
     const bool late_sync = QS == 1 && wave >= 4;
-#define CDM_ATTN_STEP(SCUR, SNEXT)                                                                              \
+#define CDM_ATTN_STEP(SCUR, SNEXT, NEEDMAX)                                                                     \
     {                                                                                                           \
         const int k_fill = ks_cur;                              /* slot of K(j)   == j % 3     */               \
         const int k_next2 = ks_next == 2 ? 0 : ks_next + 1;     /* slot of K(j+2) == (j+2) % 3 */               \
@@ -463,18 +508,27 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QS];                                                                                         \
         _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },                       \
+        pipe_step<HD, QS, NEEDMAX>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },         \
                           sk + ks_next * TILE_BYTES, sv + v_cur * TILE_BYTES, sk + k_next2 * TILE_BYTES, qf, kw, \
-                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 == NT), nvalid);  \
+                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 >= NT), nvalid);  \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         if (late_sync) load_v();                                                                                \
         ks_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
-    for (int j = 0; j < NTW; ++j) {
-        CDM_ATTN_STEP(s_a, s_b)
-        if (++j >= NTW) break;
-        CDM_ATTN_STEP(s_b, s_a)
+    // wave-uniform choice; both loops take the same barriers
+    if (need_max) {
+        for (int j = 0; j < NTW; ++j) {
+            CDM_ATTN_STEP(s_a, s_b, true)
+            if (++j >= NTW) break;
+            CDM_ATTN_STEP(s_b, s_a, true)
+        }
+    } else if constexpr (BOUND) {
+        for (int j = 0; j < NTW; ++j) {
+            CDM_ATTN_STEP(s_a, s_b, false)
+            if (++j >= NTW) break;
+            CDM_ATTN_STEP(s_b, s_a, false)
+        }
     }
 #undef CDM_ATTN_STEP
     // no direct-to-LDS write may outlive the workgroup; after the barrier no wave reads the K / V rings any more and
@@ -517,8 +571,10 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
                                                       const bf16_t* __restrict__ v, int64_t ldv,
                                                       const float* __restrict__ cos, const float* __restrict__ sin,
                                                       const QkNormDev kn, char* __restrict__ kp, char* __restrict__ vp,
-                                                      int n_tokens, int n_tiles) {
+                                                      float* __restrict__ kmax, int n_tokens, int n_tiles) {
     __shared__ bf16_t tile[64][HD + 2];
+    __shared__ float wave_kmax[4];
+    float ksq_max = 0.0f;      // largest squared norm among the keys this thread has helped with
     constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
     constexpr int HALF = HD / 2;
     constexpr int TILE_BYTES = BN * HD * 2;
@@ -578,6 +634,18 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
                 k2 = make_uint4(o2[0], o2[1], o2[2], o2[3]);
             }
         }
+        {   // squared norm of the key as stored (rounded to bf16): the CPR/2 consecutive threads of a token hold it
+            const uint32_t w1[4] = {k1.x, k1.y, k1.z, k1.w}, w2[4] = {k2.x, k2.y, k2.z, k2.w};
+            float ss = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float a0 = bf16lo(w1[j]), a1 = bf16hi(w1[j]), b0 = bf16lo(w2[j]), b1 = bf16hi(w2[j]);
+                ss += a0 * a0 + a1 * a1 + b0 * b0 + b1 * b1;
+            }
+#pragma unroll
+            for (int off = 1; off < CPR / 2; off <<= 1) ss += __shfl_xor(ss, off, 64);
+            ksq_max = fmaxf(ksq_max, ss);
+        }
         *reinterpret_cast<uint4*>(kt + (ch * 64 + r) * 16) = k1;                  // chunk-major K image
         *reinterpret_cast<uint4*>(kt + ((ch + CPR / 2) * 64 + r) * 16) = k2;
         uint32_t* d1 = reinterpret_cast<uint32_t*>(&tile[r][ch * 8]);
@@ -585,7 +653,12 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
         d1[0] = v1.x; d1[1] = v1.y; d1[2] = v1.z; d1[3] = v1.w;
         d2[0] = v2.x; d2[1] = v2.y; d2[2] = v2.z; d2[3] = v2.w;
     }
+    ksq_max = wave_max(ksq_max);
+    if ((threadIdx.x & 63) == 0) wave_kmax[threadIdx.x >> 6] = ksq_max;
     __syncthreads();
+    if (threadIdx.x == 0)
+        kmax[(int64_t)head * n_tiles + tile_idx] =
+            sqrtf(fmaxf(fmaxf(wave_kmax[0], wave_kmax[1]), fmaxf(wave_kmax[2], wave_kmax[3])));
     for (int idx = threadIdx.x; idx < HD * 8; idx += 256) {
         const int row = idx % HD, c = idx / HD;                            // channel row, key chunk
         uint32_t w[4];
@@ -599,6 +672,9 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
 inline int64_t pad_tokens(int64_t n) { return (n + BN - 1) / BN * BN; }
 inline int64_t image_bytes(int64_t n_tokens, int n_heads, int head_dim) {      // one packed tensor
     return pad_tokens(n_tokens) * n_heads * head_dim * 2;
+}
+inline int64_t kmax_bytes(int64_t n_tokens, int n_heads) {      // one float per (head, tile), padded to 16 bytes
+    return (pad_tokens(n_tokens) / BN * n_heads * 4 + 15) / 16 * 16;
 }
 
 // host view of the optional QK-norm argument -> kernel descriptor (which = 0: q weights, 1: k weights)
@@ -635,10 +711,10 @@ int32_t check_attn_common(const char* who, int64_t n_tokens, int32_t n_heads, in
 
 }  // namespace
 
-// workspace = [Kp | Vp]: the two tile images; n_heads counts K / V heads
+// workspace = [Kp | Vp | kmax]: the two tile images and the largest key norm of every tile; n_heads counts K / V heads
 extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
     if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0) return 0;
-    return 2 * image_bytes(n_tokens, n_heads, head_dim);
+    return 2 * image_bytes(n_tokens, n_heads, head_dim) + kmax_bytes(n_tokens, n_heads);
 }
 
 extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
@@ -666,10 +742,10 @@ extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void*
     hipStream_t st = (hipStream_t)stream;
     if (head_dim == 128)
         pack_kv_kernel<128><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, kn, ws, ws + img,
-                                                  (int)n_tokens, n_tiles);
+                                                  (float*)(ws + 2 * img), (int)n_tokens, n_tiles);
     else
         pack_kv_kernel<64><<<grid, 256, 0, st>>>((const bf16_t*)k, ldk, (const bf16_t*)v, ldv, cos, sin, kn, ws, ws + img,
-                                                 (int)n_tokens, n_tiles);
+                                                 (float*)(ws + 2 * img), (int)n_tokens, n_tiles);
     return cdm_check_launch("attn_pack_kv");
 }
 
@@ -703,8 +779,10 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     PackedParams p;
     p.q = (const bf16_t*)q; p.ldq = ldq;
     p.kp = (const char*)workspace; p.vp = (const char*)workspace + img;
+    p.kmax = (const float*)((const char*)workspace + 2 * img);
     p.kp_prefix = (const char*)prefix_workspace;
     p.vp_prefix = (const char*)prefix_workspace + image_bytes(n_prefix_tokens, n_kv_heads, head_dim);
+    p.kmax_prefix = (const float*)((const char*)prefix_workspace + 2 * image_bytes(n_prefix_tokens, n_kv_heads, head_dim));
     p.n_prefix_tiles = (int)(n_prefix_tokens / BN);
     p.causal_prefix = (int)causal_prefix;
     p.o = (bf16_t*)o; p.ldo = ldo;
@@ -718,14 +796,16 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     CDM_REQUIRE(nwg < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd_packed: grid too large");
     dim3 grid((unsigned)nwg);
     hipStream_t st = (hipStream_t)stream;
-    // variant 0 = 32 query rows per wave (8 waves, two per SIMD); 1 = 64 query rows per wave (4 waves)
-    if (cdm_get_variant(0) == 1) {
-        if (head_dim == 128) attn_fwd_pipe_kernel<128, 2><<<grid, 256, 0, st>>>(p);
-        else attn_fwd_pipe_kernel<64, 2><<<grid, 256, 0, st>>>(p);
-    } else {
-        if (head_dim == 128) attn_fwd_pipe_kernel<128, 1><<<grid, 512, 0, st>>>(p);
-        else attn_fwd_pipe_kernel<64, 1><<<grid, 512, 0, st>>>(p);
-    }
+    // variant 0 = 32 query rows per wave (8 waves, two per SIMD), row maxima dropped where the norm bound allows;
+    // cross-checks: 1 = 64 query rows per wave (4 waves), 2 = variant 0 with the row maxima always taken
+    const int variant = cdm_get_variant(0);
+#define CDM_ATTN_LAUNCH(QS_, BOUND_, THREADS)                                                   \
+    if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_, BOUND_><<<grid, THREADS, 0, st>>>(p);  \
+    else attn_fwd_pipe_kernel<64, QS_, BOUND_><<<grid, THREADS, 0, st>>>(p)
+    if (variant == 1) { CDM_ATTN_LAUNCH(2, false, 256); }
+    else if (variant == 2) { CDM_ATTN_LAUNCH(1, false, 512); }
+    else { CDM_ATTN_LAUNCH(1, true, 512); }
+#undef CDM_ATTN_LAUNCH
     return cdm_check_launch("attn_fwd_packed");
 }
 

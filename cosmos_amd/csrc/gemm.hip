@@ -46,7 +46,7 @@ struct GemmParams {
     const void* A; int64_t lda;          // operand strides in BYTES
     int64_t ldw;
     const float* sa;                     // fp8 only: per-row scale of A, indexed by the global row
-    bf16_t* C; int64_t ldc;
+    bf16_t* C; int64_t ldc;              // fp32 storage behind the same pointers for CDM_EPI_GATE_RESIDUAL_F32
     int N, K;
     const bf16_t* R; int64_t ldr;
     const float* cos; const float* sin;
@@ -179,14 +179,15 @@ __device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) 
 
 constexpr int kStagePitch = 256 + 16;      // bytes per staged row (16-byte multiple; the pad spreads rows over banks)
 
-// wave-private staging area -> C: COLS (128 or 64) bf16 columns of 128 rows, whole rows per store instruction
-template <int COLS>
+// wave-private staging area -> C: COLS (128 or 64) columns of ESIZE bytes (2 = bf16, 4 = fp32) of 128 rows, whole rows
+// per store instruction
+template <int COLS, int ESIZE = 2>
 __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, const char* stage, int row0, int col0, int lane) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
-    constexpr int LPR = COLS / 8;                // lanes per row (16 bytes each)
+    constexpr int LPR = COLS * ESIZE / 16;       // lanes per row (16 bytes each)
     constexpr int RPI = 64 / LPR;                // rows per instruction
     const int rl = lane / LPR, ch = lane % LPR;
-    const int col = col0 + ch * 8;
+    const int col = col0 + ch * (16 / ESIZE);
 #pragma unroll
     for (int it = 0; it < 128 / RPI; ++it) {
         const int rloc = it * RPI + rl;
@@ -197,7 +198,8 @@ __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, con
         if (row < t.m_end && col < p.N) {
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
             const u32x4 vv = {v.x, v.y, v.z, v.w};
-            __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(p.C + (int64_t)row * p.ldc + col));
+            __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.C) +
+                                                                     ((int64_t)row * p.ldc + col) * ESIZE));
         }
     }
 }
@@ -246,6 +248,42 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
         return;
     }
     const int col_base = n0 + wn * 128 + 4 * kh;
+    if (EPI == CDM_EPI_GATE_RESIDUAL_F32) {
+        // the residual stream in fp32: R and C are float rows (in place when they coincide).  A wave's 128 x 128
+        // result goes through its staging area 64 columns (256 bytes per row) at a time.
+        float* C = reinterpret_cast<float*>(p.C);
+        const float* R = reinterpret_cast<const float*>(p.R);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) {
+                const int row = row_base + mi * 32;
+                if (row >= t.m_end) continue;
+                const float sr = FP8 ? p.sa[row] : 1.0f;
+#pragma unroll
+                for (int nj = 0; nj < 2; ++nj)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int ni = 2 * h + nj;
+                        const int col = col_base + ni * 32 + 8 * g;
+                        if (col >= p.N) continue;
+                        const float4 r4 = *reinterpret_cast<const float4*>(R + (int64_t)row * p.ldr + col);
+                        float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
+                        if (t.gate) g4 = *reinterpret_cast<const float4*>(t.gate + col);
+                        if (FP8) {
+                            const float4 w4 = *reinterpret_cast<const float4*>(t.sw + col);
+                            g4.x *= sr * w4.x; g4.y *= sr * w4.y; g4.z *= sr * w4.z; g4.w *= sr * w4.w;
+                        }
+                        const float4 o = make_float4(r4.x + g4.x * acc[mi][ni][4 * g], r4.y + g4.y * acc[mi][ni][4 * g + 1],
+                                                     r4.z + g4.z * acc[mi][ni][4 * g + 2], r4.w + g4.w * acc[mi][ni][4 * g + 3]);
+                        if (stage) *reinterpret_cast<float4*>(stage + (mi * 32 + r32) * kStagePitch + (nj * 32 + 8 * g + 4 * kh) * 4) = o;
+                        else *reinterpret_cast<float4*>(C + (int64_t)row * p.ldc + col) = o;
+                    }
+            }
+            if (stage) copy_out<64, 4>(p, t, stage, m0 + wm * 128, n0 + wn * 128 + 64 * h, lane);
+        }
+        return;
+    }
     const bool rope = EPI == CDM_EPI_ROPE_QK && n0 + wn * 128 < p.rope_cols;   // wave-uniform: whole heads of Q or K
     const int half = p.head_dim >> 1;
 #pragma unroll
@@ -573,7 +611,7 @@ int32_t validate(const char* who, int esize, const void* A, int64_t lda, const v
     CDM_REQUIRE(A && W && C, CDM_ERR_BAD_ARG, "%s: null pointer", who);
     CDM_REQUIRE(M >= 0 && N > 0 && K > 0, CDM_ERR_BAD_ARG, "%s: bad sizes M=%lld N=%lld K=%lld", who, (long long)M,
                 (long long)N, (long long)K);
-    CDM_REQUIRE(epi >= CDM_EPI_NONE && epi <= CDM_EPI_ROPE_QK, CDM_ERR_BAD_ARG, "%s: unknown epilogue %d", who, epi);
+    CDM_REQUIRE(epi >= CDM_EPI_NONE && epi <= CDM_EPI_GATE_RESIDUAL_F32, CDM_ERR_BAD_ARG, "%s: unknown epilogue %d", who, epi);
     CDM_REQUIRE(K % kmult == 0, CDM_ERR_BAD_SHAPE, "%s: K=%lld must be a multiple of %lld", who, (long long)K,
                 (long long)kmult);
     CDM_REQUIRE(N % 8 == 0, CDM_ERR_BAD_SHAPE, "%s: N=%lld must be a multiple of 8", who, (long long)N);
@@ -587,7 +625,7 @@ int32_t validate(const char* who, int esize, const void* A, int64_t lda, const v
     CDM_REQUIRE(ldc % 8 == 0, CDM_ERR_BAD_ALIGN, "%s: ldc=%lld must be a multiple of 8 elements", who, (long long)ldc);
     if (epi == CDM_EPI_SWIGLU)
         CDM_REQUIRE(W2 && cdm_aligned16(W2), CDM_ERR_BAD_ARG, "%s: SWIGLU needs an aligned W2 (up_proj)", who);
-    if (epi == CDM_EPI_GATE_RESIDUAL)
+    if (epi == CDM_EPI_GATE_RESIDUAL || epi == CDM_EPI_GATE_RESIDUAL_F32)
     {
         CDM_REQUIRE(R && ldr >= N, CDM_ERR_BAD_ARG, "%s: GATE_RESIDUAL needs R with ldr >= N", who);
         CDM_REQUIRE(cdm_aligned16(R) && ldr % 8 == 0, CDM_ERR_BAD_ALIGN,
@@ -640,6 +678,7 @@ int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epi
             case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;
             case CDM_EPI_SWIGLU: CDM_LAUNCH(CDM_EPI_SWIGLU); break;
             case CDM_EPI_GATE_RESIDUAL: CDM_LAUNCH(CDM_EPI_GATE_RESIDUAL); break;
+            case CDM_EPI_GATE_RESIDUAL_F32: CDM_LAUNCH(CDM_EPI_GATE_RESIDUAL_F32); break;
             default: CDM_LAUNCH(CDM_EPI_ROPE_QK); break;
         }
 #undef CDM_LAUNCH

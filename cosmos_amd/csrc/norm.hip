@@ -39,10 +39,10 @@ __device__ __forceinline__ float block_reduce(float v, float (*slot)[4], int& pa
     return IS_MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
 }
 
-// MAXC = chunks of 8 channels per thread (d <= 2048 * MAXC)
-template <int MAXC, bool QUANT>
+// MAXC = chunks of 8 channels per thread (d <= 2048 * MAXC); XF32: the input rows are fp32 instead of bf16
+template <int MAXC, bool QUANT, bool XF32>
 __global__ __launch_bounds__(kThreads) void adaln_rmsnorm_kernel(
-    const uint4* __restrict__ x, const uint4* __restrict__ w, const float* __restrict__ shift,
+    const void* __restrict__ x, const uint4* __restrict__ w, const float* __restrict__ shift,
     const float* __restrict__ scale, void* __restrict__ y, float* __restrict__ s_tok, int64_t n_tokens,
     int d, float eps) {
     __shared__ float slot_sum[2][4];
@@ -72,13 +72,16 @@ __global__ __launch_bounds__(kThreads) void adaln_rmsnorm_kernel(
 
     const float inv_d = 1.0f / (float)d;
     // the next row's loads are issued before the current row is reduced, so a workgroup always has a row in flight
-    uint4 raw[MAXC];
+    // XF32 (residual stream kept in fp32): a chunk of 8 channels is 32 bytes of the row instead of 16
+    uint4 raw[MAXC][XF32 ? 2 : 1];
     auto fetch = [&](int64_t row) {
-        const uint4* xr = x + row * nchunk;
+        const uint4* xr = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(x) + row * (int64_t)d * (XF32 ? 4 : 2));
 #pragma unroll
         for (int c = 0; c < MAXC; ++c) {
             const int idx = c * kThreads + tid;
-            raw[c] = idx < nchunk ? xr[idx] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int h = 0; h < (XF32 ? 2 : 1); ++h)
+                raw[c][h] = idx < nchunk ? xr[(XF32 ? 2 : 1) * idx + h] : make_uint4(0, 0, 0, 0);
         }
     };
     if ((int64_t)blockIdx.x < n_tokens) fetch(blockIdx.x);
@@ -87,7 +90,15 @@ __global__ __launch_bounds__(kThreads) void adaln_rmsnorm_kernel(
         float ss = 0.0f;
 #pragma unroll
         for (int c = 0; c < MAXC; ++c) {
-            unpack8(raw[c], xv[c]);
+            if constexpr (XF32) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    xv[c][4 * h + 0] = __uint_as_float(raw[c][h].x); xv[c][4 * h + 1] = __uint_as_float(raw[c][h].y);
+                    xv[c][4 * h + 2] = __uint_as_float(raw[c][h].z); xv[c][4 * h + 3] = __uint_as_float(raw[c][h].w);
+                }
+            } else {
+                unpack8(raw[c][0], xv[c]);
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) ss += xv[c][i] * xv[c][i];
         }
@@ -178,15 +189,15 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(const bf16_t* __re
     }
 }
 
-template <bool QUANT>
+template <bool QUANT, bool XF32>
 int32_t launch_norm(const void* x, const void* w, const float* shift, const float* scale, void* y, float* s_tok,
                     int64_t n_tokens, int64_t d, float eps, hipStream_t st) {
     const int64_t max_blocks = 256 * 8;
     const int grid = (int)(n_tokens < max_blocks ? n_tokens : max_blocks);
     const int chunks = (int)((d / 8 + kThreads - 1) / kThreads);
 #define CDM_NORM_LAUNCH(C)                                                                                  \
-    adaln_rmsnorm_kernel<C, QUANT><<<grid, kThreads, 0, st>>>((const uint4*)x, (const uint4*)w, shift, scale, y, \
-                                                              s_tok, n_tokens, (int)d, eps)
+    adaln_rmsnorm_kernel<C, QUANT, XF32><<<grid, kThreads, 0, st>>>(x, (const uint4*)w, shift, scale, y, s_tok, \
+                                                                    n_tokens, (int)d, eps)
     if (chunks <= 1) CDM_NORM_LAUNCH(1);
     else if (chunks == 2) CDM_NORM_LAUNCH(2);
     else CDM_NORM_LAUNCH(4);
@@ -212,7 +223,16 @@ extern "C" int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const fl
     if (rc) return rc;
     if ((rc = cdm_require_device())) return rc;
     if (n_tokens == 0) return CDM_OK;
-    return launch_norm<false>(x, w, shift, scale, y, nullptr, n_tokens, d, eps, (hipStream_t)stream);
+    return launch_norm<false, false>(x, w, shift, scale, y, nullptr, n_tokens, d, eps, (hipStream_t)stream);
+}
+
+extern "C" int32_t cdm_adaln_rmsnorm_f32(const float* x, const void* w, const float* shift, const float* scale,
+                                         void* y, int64_t n_tokens, int64_t d, float eps, void* stream) {
+    int32_t rc = check_norm_args(x, w, y, n_tokens, d);
+    if (rc) return rc;
+    if ((rc = cdm_require_device())) return rc;
+    if (n_tokens == 0) return CDM_OK;
+    return launch_norm<false, true>(x, w, shift, scale, y, nullptr, n_tokens, d, eps, (hipStream_t)stream);
 }
 
 extern "C" int32_t cdm_adaln_rmsnorm_quant_e4m3(const void* x, const void* w, const float* shift,
@@ -223,7 +243,18 @@ extern "C" int32_t cdm_adaln_rmsnorm_quant_e4m3(const void* x, const void* w, co
     CDM_REQUIRE(s_tok, CDM_ERR_BAD_ARG, "adaln_rmsnorm_quant: null s_tok");
     if ((rc = cdm_require_device())) return rc;
     if (n_tokens == 0) return CDM_OK;
-    return launch_norm<true>(x, w, shift, scale, yq, s_tok, n_tokens, d, eps, (hipStream_t)stream);
+    return launch_norm<true, false>(x, w, shift, scale, yq, s_tok, n_tokens, d, eps, (hipStream_t)stream);
+}
+
+extern "C" int32_t cdm_adaln_rmsnorm_f32_quant_e4m3(const float* x, const void* w, const float* shift,
+                                                    const float* scale, void* yq, float* s_tok, int64_t n_tokens,
+                                                    int64_t d, float eps, void* stream) {
+    int32_t rc = check_norm_args(x, w, yq, n_tokens, d);
+    if (rc) return rc;
+    CDM_REQUIRE(s_tok, CDM_ERR_BAD_ARG, "adaln_rmsnorm_quant: null s_tok");
+    if ((rc = cdm_require_device())) return rc;
+    if (n_tokens == 0) return CDM_OK;
+    return launch_norm<true, true>(x, w, shift, scale, yq, s_tok, n_tokens, d, eps, (hipStream_t)stream);
 }
 
 extern "C" int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, float* s, int64_t rows, int64_t cols,

@@ -63,10 +63,15 @@ class Workspace:
     """Caller-owned scratch tensors of one (n_tokens, d, hidden) shape, reused by every block."""
 
     def __init__(self, n: int, d: int, hidden: int, n_heads: int, head_dim: int, device,
-                 n_kv_heads: Optional[int] = None):
+                 n_kv_heads: Optional[int] = None, fp8: bool = False):
         bf = dict(dtype=torch.bfloat16, device=device)
         n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
-        self.n, self.d, self.hidden = n, d, hidden
+        self.n, self.d, self.hidden, self.fp8 = n, d, hidden, fp8
+        if fp8:     # e4m3 operands of the four linears and their per-token scales
+            q8, f32 = dict(dtype=ops.FP8_DTYPE, device=device), dict(dtype=torch.float32, device=device)
+            self.yq, self.ys = torch.empty((n, d), **q8), torch.empty((n,), **f32)
+            self.oq, self.os = torch.empty((n, d), **q8), torch.empty((n,), **f32)
+            self.hq, self.hs = torch.empty((n, hidden), **q8), torch.empty((n,), **f32)
         self.y = torch.empty((n, d), **bf)
         self.qkv = torch.empty((n, d + 2 * n_kv_heads * head_dim), **bf)       # [Q | K | V] columns
         self.attn_out = torch.empty((n, d), **bf)
@@ -74,8 +79,8 @@ class Workspace:
         self.attn_ws = torch.empty((max(ops.attn_workspace_bytes(n, n_kv_heads, head_dim), 16),), dtype=torch.uint8,
                                    device=device)
 
-    def fits(self, n: int, d: int, hidden: int) -> bool:
-        return (self.n, self.d, self.hidden) == (n, d, hidden)
+    def fits(self, n: int, d: int, hidden: int, fp8: bool = False) -> bool:
+        return (self.n, self.d, self.hidden) == (n, d, hidden) and (self.fp8 or not fp8)
 
 
 class DMAttnProcessor:
@@ -106,6 +111,8 @@ class DMAttnProcessor:
         is the buffer this call packs its own K/V into (kept by the caller when it wants to reuse them)."""
         if attention_mask is not None:
             raise NotImplementedError("masks are selected with causal_prefix; attention_mask must be None")
+        if not isinstance(attn, _AttentionCore):
+            attn = adopt_attention(attn)      # a diffusers-style attention module: fused views, built once
         if image_rotary_emb is None:
             raise ValueError("image_rotary_emb=(cos, sin) is required")
         batched = hidden_states.dim() == 3
@@ -155,7 +162,7 @@ class DMAttnProcessor:
                 ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin,
                               qk_norm=qkn, **mask_kw)
         if attn.fp8:
-            oq, so = ops.quant_rows(o)
+            oq, so = ops.quant_rows(o, ws.oq, ws.os) if ws is not None and ws.fp8 else ops.quant_rows(o)
         else:
             oq, so = o, None
         if residual is not None:
@@ -172,7 +179,127 @@ class DMAttnProcessor:
         return out.unsqueeze(0) if batched else out
 
 
-class DMAttention(nn.Module):
+class _AttentionCore:
+    """What the processor needs of an attention module: geometry (d_model, n_heads, n_kv_heads, head_dim, n_branches),
+    per-branch fused QKV / output weights (``qkv_weight[b]``, ``out_weight[b]``), optional per-branch QK-RMSNorm rows
+    (``norm_q_weight`` / ``norm_k_weight`` [n_branches, head_dim] fp32) and optional e4m3 copies (``_q``)."""
+
+    def _weights(self, which: str):
+        return self.qkv_weight if which == "qkv" else self.out_weight
+
+    def quantize_(self) -> None:
+        """Offline per-output-channel e4m3 quantisation of this module's weights (fp8 variant)."""
+        self._q["qkv"] = [ops.quant_rows(_data(w)) for w in self.qkv_weight]
+        self._q["out"] = [ops.quant_rows(_data(w)) for w in self.out_weight]
+
+    def qk_norm_args(self, segments: Sequence[Segment]):
+        """(q_weight, k_weight, seg_ends, eps) for ``ops.attention``: one weight row per token segment."""
+        if not self.qk_norm:
+            return None
+        branches = [b for (_, _, b, _) in segments]
+        ends = [s0 + ln for (s0, ln, _, _) in segments]
+        qw, kw = _data(self.norm_q_weight), _data(self.norm_k_weight)
+        if branches != list(range(self.n_branches)):
+            idx = torch.tensor(branches, device=qw.device)
+            qw, kw = qw.index_select(0, idx).contiguous(), kw.index_select(0, idx).contiguous()
+        return qw, kw, ends, self.qk_eps
+
+    def _linear(self, a: torch.Tensor, sa: Optional[torch.Tensor], which: str, segments: Sequence[Segment], *,
+                out: torch.Tensor, epilogue: str, residual=None, gates=None, cos=None, sin=None, rope_cols=0,
+                head_dim=0) -> None:
+        _routed_linear(a, sa, self._weights(which), self._q.get(which) if self.fp8 else None, None, segments, out=out,
+                       epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
+                       head_dim=head_dim)
+
+
+def _data(t):
+    return t.data if isinstance(t, nn.Parameter) else t
+
+
+class AdoptedAttention(_AttentionCore):
+    """The HIP path's view of a diffusers-style joint-attention module that carries the sub-module names of the
+    reference's attention layers (transformers models/cosmos3_omni/modeling_cosmos3_omni.py:41-46): ``to_q / to_k /
+    to_v / to_out[0]`` (AR branch: the context tokens, branch 0), ``add_q_proj / add_k_proj / add_v_proj /
+    to_add_out`` (DM branch: the generator tokens, branch 1), optional ``norm_q / norm_k / norm_added_q /
+    norm_added_k``.
+
+    The three projections of a branch are concatenated ONCE into the fused ``[d + 2 d_kv, d]`` weight the QKV GEMM
+    reads, and the module's own ``weight`` tensors are re-pointed at row ranges of that fused tensor: one copy of the
+    weights stays alive, ``state_dict`` / ``load_state_dict`` / ``.to()`` of the module keep working on it (a
+    ``load_state_dict`` writes through the views), and the separate originals are released."""
+
+    def __init__(self, mod: nn.Module):
+        lin = lambda m: m[0] if isinstance(m, (nn.ModuleList, nn.Sequential)) else m
+        branches = [(mod.to_q, mod.to_k, mod.to_v, lin(mod.to_out))]
+        if getattr(mod, "add_q_proj", None) is not None:
+            branches.append((mod.add_q_proj, mod.add_k_proj, mod.add_v_proj, lin(mod.to_add_out)))
+        wq = mod.to_q.weight
+        if not wq.is_cuda or wq.dtype != torch.bfloat16:
+            raise RuntimeError("the HIP path needs the attention module on the GPU in bfloat16 (pipe.to('cuda'), bf16)")
+        self.d_model = wq.shape[1]
+        heads = getattr(mod, "heads", None) or getattr(mod, "num_heads", None) or getattr(mod, "n_heads", None)
+        if not heads:
+            raise ValueError("cannot tell the number of heads of this attention module (no .heads attribute)")
+        self.n_heads = int(heads)
+        if wq.shape[0] != self.d_model or self.d_model % self.n_heads:
+            raise ValueError("query projection must be square with a width divisible by the number of heads")
+        self.head_dim = self.d_model // self.n_heads
+        dkv = mod.to_k.weight.shape[0]
+        if dkv % self.head_dim or self.n_heads % (dkv // self.head_dim):
+            raise ValueError("K/V projection width does not give a whole number of heads that divides the query heads")
+        self.n_kv_heads = dkv // self.head_dim
+        self.n_branches, self.fp8, self._q = len(branches), False, {}
+        self.qkv_weight, self.out_weight, self._views = [], [], []
+        d = self.d_model
+        for (q, k, v, o) in branches:
+            for m in (q, k, v, o):
+                if getattr(m, "bias", None) is not None:
+                    raise NotImplementedError("projections with a bias are not supported by the fused kernels")
+            if q.weight.shape != (d, d) or k.weight.shape != (dkv, d) or v.weight.shape != (dkv, d) or o.weight.shape != (d, d):
+                raise ValueError("projection shapes do not match [d, d] / [d_kv, d] / [d_kv, d] / [d, d]")
+            fused = torch.cat([q.weight.data, k.weight.data, v.weight.data], dim=0).contiguous()
+            q.weight.data, k.weight.data, v.weight.data = fused[:d], fused[d:d + dkv], fused[d + dkv:]
+            self.qkv_weight.append(fused)
+            self.out_weight.append(o.weight.data if o.weight.data.is_contiguous() else o.weight.data.contiguous())
+            self._views.append((q.weight, k.weight, v.weight, o.weight))
+        nq = [getattr(mod, n, None) for n in ("norm_q", "norm_added_q")][:self.n_branches]
+        nk = [getattr(mod, n, None) for n in ("norm_k", "norm_added_k")][:self.n_branches]
+        self.qk_norm = all(m is not None and getattr(m, "weight", None) is not None for m in nq + nk)
+        self.qk_eps = 1e-6
+        if self.qk_norm:
+            self._norm_mods = (nq, nk)
+            self.qk_eps = float(getattr(nq[0], "eps", getattr(nq[0], "variance_epsilon", 1e-6)))
+            self.norm_q_weight = torch.stack([m.weight.data.float() for m in nq]).contiguous()
+            self.norm_k_weight = torch.stack([m.weight.data.float() for m in nk]).contiguous()
+            self._norm_seen = [(m.weight.data_ptr(), m.weight._version) for m in nq + nk]
+
+    def still_valid(self) -> bool:
+        """False once some weight of the module has been replaced (a new tensor assigned, moved to another device)."""
+        d, dkv = self.d_model, self.n_kv_heads * self.head_dim
+        for fused, o, (q, k, v, ow) in zip(self.qkv_weight, self.out_weight, self._views):
+            es = fused.element_size()
+            if (q.data_ptr(), k.data_ptr(), v.data_ptr()) != (fused.data_ptr(), fused.data_ptr() + d * d * es,
+                                                              fused.data_ptr() + (d + dkv) * d * es):
+                return False
+            if ow.data_ptr() != o.data_ptr() and ow.data.is_contiguous():
+                return False
+        if self.qk_norm:      # the fp32 norm rows are copies: rebuilt when a norm weight was replaced or written to
+            nq, nk = self._norm_mods
+            if [(m.weight.data_ptr(), m.weight._version) for m in nq + nk] != self._norm_seen:
+                return False
+        return True
+
+
+def adopt_attention(mod: nn.Module) -> AdoptedAttention:
+    """The cached ``AdoptedAttention`` of a diffusers-style attention module (built at the first call)."""
+    ad = mod.__dict__.get("_cdm_adopted")
+    if ad is None or not ad.still_valid():
+        ad = AdoptedAttention(mod)
+        mod.__dict__["_cdm_adopted"] = ad       # not a sub-module: the module's state_dict is unchanged
+    return ad
+
+
+class DMAttention(nn.Module, _AttentionCore):
     """Attention module of one MoT layer: per-branch projections around one shared attention."""
 
     def __init__(self, d_model: int, n_heads: int, head_dim: int, n_branches: int = 1, fp8: bool = False,
@@ -205,33 +332,6 @@ class DMAttention(nn.Module):
 
     def set_processor(self, processor) -> None:
         self.processor = processor
-
-    def quantize_(self) -> None:
-        """Offline per-output-channel e4m3 quantisation of this module's weights (fp8 variant)."""
-        self._q["qkv"] = [ops.quant_rows(w.data) for w in self.qkv_weight]
-        self._q["out"] = [ops.quant_rows(w.data) for w in self.out_weight]
-
-    def _weights(self, which: str):
-        return self.qkv_weight if which == "qkv" else self.out_weight
-
-    def qk_norm_args(self, segments: Sequence[Segment]):
-        """(q_weight, k_weight, seg_ends, eps) for ``ops.attention``: one weight row per token segment."""
-        if not self.qk_norm:
-            return None
-        branches = [b for (_, _, b, _) in segments]
-        ends = [s0 + ln for (s0, ln, _, _) in segments]
-        qw, kw = self.norm_q_weight.data, self.norm_k_weight.data
-        if branches != list(range(self.n_branches)):
-            idx = torch.tensor(branches, device=qw.device)
-            qw, kw = qw.index_select(0, idx).contiguous(), kw.index_select(0, idx).contiguous()
-        return qw, kw, ends, self.qk_eps
-
-    def _linear(self, a: torch.Tensor, sa: Optional[torch.Tensor], which: str, segments: Sequence[Segment], *,
-                out: torch.Tensor, epilogue: str, residual=None, gates=None, cos=None, sin=None, rope_cols=0,
-                head_dim=0) -> None:
-        _routed_linear(a, sa, self._weights(which), self._q.get(which) if self.fp8 else None, None, segments, out=out,
-                       epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
-                       head_dim=head_dim)
 
     def forward(self, hidden_states, encoder_hidden_states=None, attention_mask=None, image_rotary_emb=None, **kw):
         return self.processor(self, hidden_states, encoder_hidden_states=encoder_hidden_states,
@@ -307,15 +407,16 @@ class DMBlock(nn.Module):
         m = self.adaLN_modulation(torch.nn.functional.silu(c)).float().reshape(-1)
         return tuple(t.contiguous() for t in m.chunk(6))
 
-    def _norm(self, x, weights, shift, scale, segments, y):
-        """Per-branch adaLN-RMSNorm into y (bf16), or into fresh (e4m3, scale) tensors for the fp8 variant."""
+    def _norm(self, x, weights, shift, scale, segments, ws):
+        """Per-branch adaLN-RMSNorm of x (bf16 or fp32) into the workspace: y (bf16), or (e4m3, per-token scale) for
+        the fp8 variant."""
         if not self.fp8:
+            y = ws.y
             for (s0, ln, b, modulated) in segments:
                 ops.adaln_rmsnorm(x[s0:s0 + ln], weights[b], shift if modulated else None, scale if modulated else None,
                                   self.eps, out=y[s0:s0 + ln])
             return y, None
-        yq = torch.empty(x.shape, dtype=ops.FP8_DTYPE, device=x.device)
-        st = torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)
+        yq, st = ws.yq, ws.ys
         for (s0, ln, b, modulated) in segments:
             ops.adaln_rmsnorm_quant(x[s0:s0 + ln], weights[b], shift if modulated else None,
                                     scale if modulated else None, self.eps, out_q=yq[s0:s0 + ln], out_s=st[s0:s0 + ln])
@@ -326,6 +427,8 @@ class DMBlock(nn.Module):
                 modality_segments: Optional[Sequence[Segment]] = None, *, inplace: bool = False,
                 modulation: Optional[Sequence[torch.Tensor]] = None, workspace: Optional[Workspace] = None,
                 causal_prefix: int = 0, prefix=None, kv_images: Optional[torch.Tensor] = None):
+        """``hidden_states`` [N, d] (or [1, N, d]) is the residual stream, bf16 or fp32; the result has its dtype (a
+        stack keeps the stream in fp32 between blocks: only the operands of the matrix products are bf16)."""
         batched = hidden_states.dim() == 3
         x = _as2d(hidden_states)
         if not inplace:
@@ -333,21 +436,22 @@ class DMBlock(nn.Module):
         n, d = x.shape
         segs = list(modality_segments) if modality_segments is not None else [(0, n, 0, True)]
         ws = workspace or self._ws
-        if ws is None or not ws.fits(n, d, self.hidden) or ws.y.device != x.device:
-            ws = Workspace(n, d, self.hidden, self.attn.n_heads, self.attn.head_dim, x.device, self.attn.n_kv_heads)
+        if ws is None or not ws.fits(n, d, self.hidden, self.fp8) or ws.y.device != x.device:
+            ws = Workspace(n, d, self.hidden, self.attn.n_heads, self.attn.head_dim, x.device, self.attn.n_kv_heads,
+                           self.fp8)
             if workspace is None:
                 self._ws = ws
         sh1, sc1, g1, sh2, sc2, g2 = modulation if modulation is not None else self.modulation(temb)
 
-        y, sy = self._norm(x, self.norm1_weight, sh1, sc1, segs, ws.y)
+        y, sy = self._norm(x, self.norm1_weight, sh1, sc1, segs, ws)
         self.attn(y, image_rotary_emb=image_rotary_emb, modality_segments=segs, residual=x, gate=g1, quant_scale=sy,
                   workspace=ws, causal_prefix=causal_prefix, prefix=prefix, kv_images=kv_images)
-        y, sy = self._norm(x, self.norm2_weight, sh2, sc2, segs, ws.y)
+        y, sy = self._norm(x, self.norm2_weight, sh2, sc2, segs, ws)
         q = self._q if self.fp8 else {}
         _routed_linear(y, sy, self.gate_weight, q.get("gate"), self.up_weight, segs, out=ws.h, epilogue="swiglu",
                        qweights2=q.get("up"))
         if self.fp8:
-            hq, sh = ops.quant_rows(ws.h)
+            hq, sh = ops.quant_rows(ws.h, ws.hq, ws.hs)
         else:
             hq, sh = ws.h, None
         gates = [g2 if modulated else None for (_, _, _, modulated) in segs]
@@ -385,7 +489,7 @@ class ContextCache:
 
 
 class DMStack(nn.Module):
-    """L blocks over the joint sequence text | video | action (diffusers transformer forward shape)."""
+    """L blocks over the joint sequence text | video | audio | action (diffusers transformer forward shape)."""
 
     def __init__(self, cfg: DMConfig, device=None, dtype=torch.bfloat16):
         super().__init__()
@@ -413,13 +517,17 @@ class DMStack(nn.Module):
             b.reset_parameters(g)
 
     def segments(self) -> List[Segment]:
-        """(start, len, branch, modulated): text uses branch 0 un-modulated; video and action are modulated."""
+        """(start, len, branch, modulated): text uses branch 0 un-modulated; the generator's modalities - video, audio,
+        action - are modulated.  Video uses the generator (DM) weight set, branch 1 of a multi-branch stack; action its
+        own third set when there is one; audio its own fourth set when there is one, else the generator's."""
         c = self.cfg
-        multi = c.n_branches > 1
+        gen = 1 if c.n_branches > 1 else 0
         segs, s = [], 0
         if c.n_text:
             segs.append((s, c.n_text, 0, False)); s += c.n_text
-        segs.append((s, c.n_video, 1 if multi else 0, True)); s += c.n_video
+        segs.append((s, c.n_video, gen, True)); s += c.n_video
+        if c.n_audio:
+            segs.append((s, c.n_audio, 3 if c.n_branches > 3 else gen, True)); s += c.n_audio
         if c.n_action:
             segs.append((s, c.n_action, min(2, c.n_branches - 1), True))
         return segs
@@ -427,7 +535,7 @@ class DMStack(nn.Module):
     def rotary(self, device) -> Tuple[torch.Tensor, torch.Tensor]:
         if self._rot is None or self._rot[0].device != torch.device(device):
             c = self.cfg
-            pos, _ = rotary.build_positions(c.n_text, c.grid, c.n_action)
+            pos, _ = rotary.build_positions(c.n_text, c.grid, c.n_action, c.n_audio)
             self._rot = rotary.rotary_tables(pos, c.head_dim, c.mrope_sections, c.rope_base, c.rope_layout, device)
         return self._rot
 
@@ -442,13 +550,13 @@ class DMStack(nn.Module):
             raise RuntimeError("context reuse needs the hybrid mask (DMConfig.hybrid_mask)")
         if c.n_text == 0 or c.n_text % 64:
             raise ValueError("context reuse needs a text run whose length is a positive multiple of 64")
-        x = _as2d(encoder_hidden_states).clone()
+        x = self._stream(_as2d(encoder_hidden_states))
         if x.shape != (c.n_text, c.d_model):
             raise ValueError(f"context has shape {tuple(x.shape)}, expected {(c.n_text, c.d_model)}")
         cos, sin = self.rotary(x.device)
         rot = (cos[:c.n_text].contiguous(), sin[:c.n_text].contiguous())
         segs = [(0, c.n_text, 0, False)]
-        ws = Workspace(c.n_text, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads)
+        ws = Workspace(c.n_text, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads, c.fp8)
         nbytes = ops.attn_workspace_bytes(c.n_text, c.kv_heads, c.head_dim)
         images = []
         for blk in self.blocks:
@@ -461,55 +569,70 @@ class DMStack(nn.Module):
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
                 encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
-                return_dict: bool = False, context_cache: Optional["ContextCache"] = None):
+                return_dict: bool = False, context_cache: Optional["ContextCache"] = None,
+                audio_states: Optional[torch.Tensor] = None):
         c = self.cfg
         batch = _batch_size(hidden_states, 3)
         if batch > 1:
             ts = timestep.reshape(-1)
             return _over_batch(lambda b: self.forward(hidden_states[b:b + 1], ts[b:b + 1] if ts.numel() == batch else ts,
                                                       _sample(encoder_hidden_states, b, 3, batch),
-                                                      _sample(action_states, b, 3, batch), return_dict, context_cache),
+                                                      _sample(action_states, b, 3, batch), return_dict, context_cache,
+                                                      _sample(audio_states, b, 3, batch)),
                                batch, return_dict)
         if context_cache is not None:
-            return self._forward_cached(hidden_states, timestep, action_states, return_dict, context_cache)
+            return self._forward_cached(hidden_states, timestep, action_states, return_dict, context_cache, audio_states)
         parts = []
         if c.n_text:
             if encoder_hidden_states is None:
                 raise ValueError("this configuration expects encoder_hidden_states (text context)")
             parts.append(_as2d(encoder_hidden_states))
         parts.append(_as2d(hidden_states))
-        if c.n_action:
-            if action_states is None:
-                raise ValueError("this configuration expects action_states")
-            parts.append(_as2d(action_states))
-        x = torch.cat(parts, dim=0).contiguous() if len(parts) > 1 else parts[0].clone()
+        parts += self._generator_extras(audio_states, action_states)
+        x = self._stream(torch.cat(parts, dim=0) if len(parts) > 1 else parts[0])
         if x.shape != (c.n_tokens, c.d_model):
             raise ValueError(f"joint sequence has shape {tuple(x.shape)}, expected {(c.n_tokens, c.d_model)}")
         rot = self.rotary(x.device)
         segs = self.segments()
         temb = self.time_embedder(timestep.reshape(-1)[:1])
-        if self._ws is None or not self._ws.fits(c.n_tokens, c.d_model, c.hidden) or self._ws.y.device != x.device:
-            self._ws = Workspace(c.n_tokens, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads)
+        if self._ws is None or not self._ws.fits(c.n_tokens, c.d_model, c.hidden, c.fp8) or self._ws.y.device != x.device:
+            self._ws = Workspace(c.n_tokens, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads, c.fp8)
         for blk in self.blocks:
             blk(x, temb, rot, segs, inplace=True, workspace=self._ws, causal_prefix=c.n_text if c.hybrid_mask else 0)
-        video = x[c.n_text:c.n_text + c.n_video]
-        out = video.unsqueeze(0) if hidden_states.dim() == 3 else video
+        return self._result(x, c.n_text, hidden_states.dim() == 3, return_dict)
+
+    def _stream(self, x: torch.Tensor) -> torch.Tensor:
+        """A private, contiguous copy of the joint sequence in the dtype the residual stream is kept in."""
+        dt = torch.float32 if self.cfg.residual_fp32 else torch.bfloat16
+        return x.to(dt).contiguous() if x.dtype != dt else x.contiguous().clone()
+
+    def _result(self, x: torch.Tensor, first_video: int, batched: bool, return_dict: bool):
+        """The video rows of the final stream as bf16 (the transformer's output dtype); "joint" is the stream itself."""
+        video = x[first_video:first_video + self.cfg.n_video].to(torch.bfloat16)
+        out = video.unsqueeze(0) if batched else video
         if return_dict:
             return {"sample": out, "joint": x}
         return (out,)
 
 
-    def _forward_cached(self, hidden_states, timestep, action_states, return_dict, cache: "ContextCache"):
+    def _generator_extras(self, audio_states, action_states) -> List[torch.Tensor]:
+        """The audio and action runs that follow the video tokens in the joint sequence."""
+        c, parts = self.cfg, []
+        for n, t, name in ((c.n_audio, audio_states, "audio_states"), (c.n_action, action_states, "action_states")):
+            if n:
+                if t is None:
+                    raise ValueError(f"this configuration expects {name}")
+                parts.append(_as2d(t))
+        return parts
+
+    def _forward_cached(self, hidden_states, timestep, action_states, return_dict, cache: "ContextCache",
+                        audio_states=None):
         c = self.cfg
         P = c.n_text
         if cache.n_tokens != P or len(cache.images) != len(self.blocks):
             raise ValueError("context cache does not belong to this stack")
-        parts = [_as2d(hidden_states)]
-        if c.n_action:
-            if action_states is None:
-                raise ValueError("this configuration expects action_states")
-            parts.append(_as2d(action_states))
-        x = torch.cat(parts, dim=0).contiguous() if len(parts) > 1 else parts[0].clone()
+        parts = [_as2d(hidden_states)] + self._generator_extras(audio_states, action_states)
+        x = self._stream(torch.cat(parts, dim=0) if len(parts) > 1 else parts[0])
         n = c.n_tokens - P
         if x.shape != (n, c.d_model):
             raise ValueError(f"generator sequence has shape {tuple(x.shape)}, expected {(n, c.d_model)}")
@@ -518,15 +641,11 @@ class DMStack(nn.Module):
             self._rot_gen = (cos[P:].contiguous(), sin[P:].contiguous())
         segs = [(s0 - P, ln, b, m) for (s0, ln, b, m) in self.segments() if s0 >= P]
         temb = self.time_embedder(timestep.reshape(-1)[:1])
-        if self._ws_gen is None or not self._ws_gen.fits(n, c.d_model, c.hidden) or self._ws_gen.y.device != x.device:
-            self._ws_gen = Workspace(n, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads)
+        if self._ws_gen is None or not self._ws_gen.fits(n, c.d_model, c.hidden, c.fp8) or self._ws_gen.y.device != x.device:
+            self._ws_gen = Workspace(n, c.d_model, c.hidden, c.n_heads, c.head_dim, x.device, c.kv_heads, c.fp8)
         for blk, img in zip(self.blocks, cache.images):
             blk(x, temb, self._rot_gen, segs, inplace=True, workspace=self._ws_gen, prefix=(img, P))
-        video = x[:c.n_video]
-        out = video.unsqueeze(0) if hidden_states.dim() == 3 else video
-        if return_dict:
-            return {"sample": out, "joint": x}
-        return (out,)
+        return self._result(x, 0, hidden_states.dim() == 3, return_dict)
 
 
 class DMTransformer(nn.Module):
@@ -534,17 +653,20 @@ class DMTransformer(nn.Module):
 
     Stack edges around ``DMStack``: patchify + ``proj_in``, the block stack, a final RMSNorm, ``proj_out`` +
     unpatchify; an optional action stream (``action_proj_in`` + ``action_modality_embed`` in, ``action_proj_out``
-    out).  The edge linears are one-off projections with K or N = patch width (64 for 16 latent channels and 1x2x2
+    out) and an optional audio stream (``audio_proj_in`` + ``audio_modality_embed`` in, ``audio_proj_out`` out: the
+    sound the reference generates with ``enable_sound``, README.md:259).  The edge linears are one-off projections with K or N = patch width (64 for 16 latent channels and 1x2x2
     patches): 0.1 % of a step's flops, they stay on the stock BLAS path like the one-row timestep MLP.  Parameter
     names follow the checkpoint keys the reference's model files attest (``proj_in``, ``proj_out``,
-    ``time_embedder``, ``action_proj_in``, ``action_proj_out``, ``action_modality_embed``); the patch order
+    ``time_embedder``, ``action_proj_in``, ``action_proj_out``, ``action_modality_embed``, ``audio_proj_in``,
+    ``audio_proj_out``, ``audio_modality_embed``); the patch order
     (channel-major inside a patch) and the un-modulated final norm are this build's choices.
     """
 
     def __init__(self, cfg: DMConfig, latent_channels: int = 16, patch: Tuple[int, int, int] = (1, 2, 2),
-                 action_dim: int = 0, device=None, dtype=torch.bfloat16):
+                 action_dim: int = 0, audio_dim: int = 0, device=None, dtype=torch.bfloat16):
         super().__init__()
         self.cfg, self.latent_channels, self.patch, self.action_dim = cfg, latent_channels, tuple(patch), action_dim
+        self.audio_dim = audio_dim
         pd = latent_channels * patch[0] * patch[1] * patch[2]
         self.stack = DMStack(cfg, device=device, dtype=dtype)
         self.proj_in = nn.Linear(pd, cfg.d_model, device=device, dtype=dtype)
@@ -557,8 +679,25 @@ class DMTransformer(nn.Module):
             self.action_proj_out = nn.Linear(cfg.d_model, action_dim, device=device, dtype=dtype)
             self.action_modality_embed = nn.Parameter(torch.zeros(cfg.d_model, device=device, dtype=dtype),
                                                       requires_grad=False)
+        if cfg.n_audio:
+            if audio_dim <= 0:
+                raise ValueError("a configuration with audio tokens needs audio_dim")
+            self.audio_proj_in = nn.Linear(audio_dim, cfg.d_model, device=device, dtype=dtype)
+            self.audio_proj_out = nn.Linear(cfg.d_model, audio_dim, device=device, dtype=dtype)
+            self.audio_modality_embed = nn.Parameter(torch.zeros(cfg.d_model, device=device, dtype=dtype),
+                                                     requires_grad=False)
         for p in self.parameters():
             p.requires_grad_(False)
+
+    def _streams(self):
+        """(name, token count, in projection, out projection, embed) of the generator's 1-D side streams, in
+        sequence order."""
+        c, out = self.cfg, []
+        if c.n_audio:
+            out.append(("audio", c.n_audio, self.audio_proj_in, self.audio_proj_out, self.audio_modality_embed))
+        if c.n_action:
+            out.append(("action", c.n_action, self.action_proj_in, self.action_proj_out, self.action_modality_embed))
+        return out
 
     @property
     def time_embedder(self):
@@ -569,7 +708,7 @@ class DMTransformer(nn.Module):
         self.stack.reset_parameters(seed)
         dev = self.proj_in.weight.device
         g = torch.Generator(device=dev).manual_seed((self.cfg.seed if seed is None else seed) + 7919)
-        mods = [self.proj_in, self.proj_out] + ([self.action_proj_in, self.action_proj_out] if self.cfg.n_action else [])
+        mods = [self.proj_in, self.proj_out] + [m for st in self._streams() for m in st[2:4]]
         for m in mods:
             m.weight.copy_((torch.randn(m.weight.shape, generator=g, device=dev) * 0.02).to(m.weight.dtype))
             m.bias.zero_()
@@ -590,52 +729,67 @@ class DMTransformer(nn.Module):
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
                 encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
-                return_dict: bool = False):
+                return_dict: bool = False, context_cache: Optional["ContextCache"] = None,
+                audio_states: Optional[torch.Tensor] = None):
         """hidden_states: latents [1, C, T*pt, H*ph, W*pw]; encoder_hidden_states: [1, n_text, d] context already in
-        model width; action_states: [1, n_action, action_dim].  Returns the velocity prediction, latents-shaped and
-        bf16 (plus the action prediction when there is an action stream)."""
+        model width; action_states: [1, n_action, action_dim]; audio_states: [1, n_audio, audio_dim].  Returns the
+        velocity prediction, latents-shaped and bf16, followed by the audio and the action prediction when those
+        streams exist (keys "sample", "audio", "action" with ``return_dict``).  ``context_cache`` (from
+        ``stack.precompute_context``, hybrid mask only) replaces ``encoder_hidden_states``: the text run's K/V are
+        reused and the forward carries only the generator tokens."""
         c = self.cfg
         batch = _batch_size(hidden_states, 5)
         if batch > 1:
             ts = timestep.reshape(-1)
             return _over_batch(lambda b: self.forward(hidden_states[b:b + 1], ts[b:b + 1] if ts.numel() == batch else ts,
                                                       _sample(encoder_hidden_states, b, 3, batch),
-                                                      _sample(action_states, b, 3, batch), return_dict),
+                                                      _sample(action_states, b, 3, batch), return_dict, context_cache,
+                                                      _sample(audio_states, b, 3, batch)),
                                batch, return_dict)
         dt = self.proj_in.weight.dtype
         tok = self.proj_in(self.patchify(hidden_states[0].to(dt)))
-        act = None
-        if c.n_action:
-            if action_states is None:
-                raise ValueError("this configuration expects action_states")
-            act = self.action_proj_in(_as2d(action_states).to(dt)) + self.action_modality_embed
-        res = self.stack(tok, timestep, encoder_hidden_states=encoder_hidden_states, action_states=act, return_dict=True)
-        joint = res["joint"]
+        given = {"audio": audio_states, "action": action_states}
+        emb = {}
+        for name, _, p_in, _, embed in self._streams():
+            if given[name] is None:
+                raise ValueError(f"this configuration expects {name}_states")
+            emb[name] = p_in(_as2d(given[name]).to(dt)) + embed
+        res = self.stack(tok, timestep, encoder_hidden_states=None if context_cache is not None else encoder_hidden_states,
+                         action_states=emb.get("action"), return_dict=True, context_cache=context_cache,
+                         audio_states=emb.get("audio"))
+        joint = res["joint"]            # with a context cache: the generator tokens only
+        first = 0 if context_cache is not None else c.n_text
         y = ops.adaln_rmsnorm(joint, self.norm_out.data, None, None, c.eps)
-        video = y[c.n_text:c.n_text + c.n_video]
+        video = y[first:first + c.n_video]
         sample = self.unpatchify(self.proj_out(video))
-        out_act = self.action_proj_out(y[c.n_text + c.n_video:]).unsqueeze(0) if c.n_action else None
+        outs, at = {"audio": None, "action": None}, first + c.n_video
+        for name, n, _, p_out, _ in self._streams():
+            outs[name] = p_out(y[at:at + n]).unsqueeze(0)
+            at += n
         if return_dict:
-            return {"sample": sample, "action": out_act}
-        return (sample,) if out_act is None else (sample, out_act)
+            return {"sample": sample, **outs}
+        return (sample,) + tuple(o for o in (outs["audio"], outs["action"]) if o is not None)
 
     # ---- checkpoint plumbing (see cosmos_amd.checkpoint)
     def _top(self):
         mods = {"proj_in": self.proj_in, "proj_out": self.proj_out, "time_embedder.linear_1": self.stack.time_embedder.linear_1,
                 "time_embedder.linear_2": self.stack.time_embedder.linear_2}
-        if self.cfg.n_action:
-            mods.update({"action_proj_in": self.action_proj_in, "action_proj_out": self.action_proj_out})
+        for name, _, p_in, p_out, _ in self._streams():
+            mods.update({f"{name}_proj_in": p_in, f"{name}_proj_out": p_out})
         t = {f"{k}.{p}": getattr(m, p) for k, m in mods.items() for p in ("weight", "bias")}
         t["norm_out.weight"] = self.norm_out
-        if self.cfg.n_action:
-            t["action_modality_embed"] = self.action_modality_embed
+        for name, _, _, _, embed in self._streams():
+            t[f"{name}_modality_embed"] = embed
         return t
 
     def top_level_keys(self) -> List[str]:
         return list(self._top())
 
     def assign_top_level(self, key: str, t: torch.Tensor) -> None:
-        self._top()[key].data.copy_(t)
+        dst = self._top()[key].data
+        if tuple(dst.shape) != tuple(t.shape):
+            raise RuntimeError(f"shape {tuple(t.shape)} does not match the model's {tuple(dst.shape)}")
+        dst.copy_(t)
 
     def export_top_level(self):
         return {k: p.data.clone() for k, p in self._top().items()}

@@ -11,10 +11,20 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from ._lib import EPI_GATE_RESIDUAL, EPI_NONE, EPI_ROPE_QK, EPI_SWIGLU
+from ._lib import EPI_GATE_RESIDUAL, EPI_GATE_RESIDUAL_F32, EPI_NONE, EPI_ROPE_QK, EPI_SWIGLU
 
 _EPI = {"none": EPI_NONE, "swiglu": EPI_SWIGLU, "gate_residual": EPI_GATE_RESIDUAL, "rope_qk": EPI_ROPE_QK}
 FP8_DTYPE = torch.float8_e4m3fn
+
+
+def _epilogue(name: str, out: torch.Tensor, residual: Optional[torch.Tensor]):
+    """(epilogue code, dtype of out / residual): "gate_residual" takes its fp32 form when ``out`` is fp32 (the
+    residual stream kept in fp32); every other epilogue writes bf16."""
+    if name == "gate_residual" and out.dtype == torch.float32:
+        if residual is None or residual.dtype != torch.float32:
+            raise TypeError("an fp32 output of the gated residual needs an fp32 residual")
+        return EPI_GATE_RESIDUAL_F32, torch.float32
+    return _EPI[name], torch.bfloat16
 
 
 def _stream() -> int:
@@ -89,18 +99,20 @@ def set_variant(op: str, variant: int) -> int:
 def adaln_rmsnorm(x: torch.Tensor, w: torch.Tensor, shift: Optional[torch.Tensor] = None,
                   scale: Optional[torch.Tensor] = None, eps: float = 1e-6,
                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y = rmsnorm(x) * w * (1 + scale) + shift; x [n, d] bf16 contiguous."""
+    """y = rmsnorm(x) * w * (1 + scale) + shift; x [n, d] contiguous, bf16 or fp32 (residual stream kept in fp32);
+    y is bf16."""
     lib = _lib.load()
     n, d = x.shape
     if not x.is_contiguous():
         raise ValueError("x must be contiguous")
-    out = torch.empty_like(x) if out is None else out
+    out = torch.empty((n, d), dtype=torch.bfloat16, device=x.device) if out is None else out
     if not out.is_contiguous() or out.shape != x.shape:
         raise ValueError("out must be a contiguous tensor of x's shape")
-    rc = lib.cdm_adaln_rmsnorm_bf16(_chk(x, "x", torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
-                                    _f32vec(shift, "shift", d), _f32vec(scale, "scale", d),
-                                    _chk(out, "out", torch.bfloat16, 2), n, d, float(eps), _stream())
-    _lib.check(rc, "cdm_adaln_rmsnorm_bf16")
+    fn = lib.cdm_adaln_rmsnorm_f32 if x.dtype == torch.float32 else lib.cdm_adaln_rmsnorm_bf16
+    rc = fn(_chk(x, "x", x.dtype if x.dtype == torch.float32 else torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
+            _f32vec(shift, "shift", d), _f32vec(scale, "scale", d), _chk(out, "out", torch.bfloat16, 2), n, d, float(eps),
+            _stream())
+    _lib.check(rc, "cdm_adaln_rmsnorm")
     return out
 
 
@@ -116,23 +128,27 @@ def adaln_rmsnorm_quant(x, w, shift=None, scale=None, eps: float = 1e-6, out_q: 
     s = torch.empty((n,), dtype=torch.float32, device=x.device) if out_s is None else out_s
     if yq.shape != (n, d) or not yq.is_contiguous() or s.shape != (n,) or not s.is_contiguous():
         raise ValueError("out_q / out_s must be contiguous [n, d] e4m3 and [n] fp32")
-    rc = lib.cdm_adaln_rmsnorm_quant_e4m3(_chk(x, "x", torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
-                                          _f32vec(shift, "shift", d), _f32vec(scale, "scale", d),
-                                          _chk(yq, "out_q", FP8_DTYPE, 2), _chk(s, "out_s", torch.float32, 1), n, d,
-                                          float(eps), _stream())
+    fn = lib.cdm_adaln_rmsnorm_f32_quant_e4m3 if x.dtype == torch.float32 else lib.cdm_adaln_rmsnorm_quant_e4m3
+    rc = fn(_chk(x, "x", x.dtype if x.dtype == torch.float32 else torch.bfloat16, 2), _chk(w, "w", torch.bfloat16, 1),
+            _f32vec(shift, "shift", d), _f32vec(scale, "scale", d), _chk(yq, "out_q", FP8_DTYPE, 2),
+            _chk(s, "out_s", torch.float32, 1), n, d, float(eps), _stream())
     _lib.check(rc, "cdm_adaln_rmsnorm_quant_e4m3")
     return yq, s
 
 
 @_timed("quant")
-def quant_rows(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Per-row e4m3 quantisation of a bf16 matrix [rows, cols] (row stride may exceed cols)."""
+def quant_rows(a: torch.Tensor, out_q: Optional[torch.Tensor] = None,
+               out_s: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row e4m3 quantisation of a bf16 matrix [rows, cols] (row stride may exceed cols); ``out_q`` / ``out_s``:
+    caller-owned [rows, cols] e4m3 and [rows] fp32 outputs."""
     lib = _lib.load()
     rows, cols = a.shape
-    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=a.device)
-    s = torch.empty((rows,), dtype=torch.float32, device=a.device)
-    rc = lib.cdm_quant_rows_e4m3(_chk(a, "a", torch.bfloat16, 2), a.stride(0), q.data_ptr(), s.data_ptr(), rows, cols,
-                                 _stream())
+    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=a.device) if out_q is None else out_q
+    s = torch.empty((rows,), dtype=torch.float32, device=a.device) if out_s is None else out_s
+    if q.shape != (rows, cols) or not q.is_contiguous() or s.shape != (rows,) or not s.is_contiguous():
+        raise ValueError("out_q / out_s must be contiguous [rows, cols] e4m3 and [rows] fp32")
+    rc = lib.cdm_quant_rows_e4m3(_chk(a, "a", torch.bfloat16, 2), a.stride(0), _chk(q, "out_q", FP8_DTYPE, 2),
+                                 _chk(s, "out_s", torch.float32, 1), rows, cols, _stream())
     _lib.check(rc, "cdm_quant_rows_e4m3")
     return q, s
 
@@ -156,9 +172,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
     if w2 is not None and w2.stride(0) != w.stride(0):
         raise ValueError("w and w2 must share a row stride")
     half = head_dim // 2 if head_dim else 0
+    epi, odt = _epilogue(epilogue, out, residual)
     rc = lib.cdm_gemm_bf16(_chk(a, "a", torch.bfloat16, 2), a.stride(0), _chk(w, "w", torch.bfloat16, 2), w.stride(0),
-                           _chk(w2, "w2", torch.bfloat16, 2), _chk(out, "out", torch.bfloat16, 2), out.stride(0),
-                           M, N, K, _EPI[epilogue], _chk(residual, "residual", torch.bfloat16, 2),
+                           _chk(w2, "w2", torch.bfloat16, 2), _chk(out, "out", odt, 2), out.stride(0),
+                           M, N, K, epi, _chk(residual, "residual", odt, 2),
                            residual.stride(0) if residual is not None else 0, _f32vec(gate, "gate", N),
                            _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols), int(head_dim),
                            _stream())
@@ -178,11 +195,12 @@ def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Ten
     if out is None:
         out = torch.empty((M, N), dtype=torch.bfloat16, device=aq.device)
     half = head_dim // 2 if head_dim else 0
+    epi, odt = _epilogue(epilogue, out, residual)
     rc = lib.cdm_gemm_fp8(_chk(aq, "aq", FP8_DTYPE, 2), aq.stride(0), _f32vec(sa, "sa", M),
                           _chk(wq, "wq", FP8_DTYPE, 2), wq.stride(0), _f32vec(sw, "sw", N),
                           _chk(w2q, "w2q", FP8_DTYPE, 2), _f32vec(sw2, "sw2", N),
-                          _chk(out, "out", torch.bfloat16, 2), out.stride(0), M, N, K, _EPI[epilogue],
-                          _chk(residual, "residual", torch.bfloat16, 2),
+                          _chk(out, "out", odt, 2), out.stride(0), M, N, K, epi,
+                          _chk(residual, "residual", odt, 2),
                           residual.stride(0) if residual is not None else 0, _f32vec(gate, "gate", N),
                           _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols), int(head_dim),
                           _stream())
@@ -213,9 +231,10 @@ def grouped_gemm(a: torch.Tensor, ws: Sequence[torch.Tensor], segments: Sequence
     I64 = C.c_int64 * n_seg
     st, ln = I64(*[int(s) for s, _ in segments]), I64(*[int(l) for _, l in segments])
     half = head_dim // 2 if head_dim else 0
+    epi, odt = _epilogue(epilogue, out, residual)
     rc = lib.cdm_grouped_gemm_bf16(_chk(a, "a", torch.bfloat16, 2), a.stride(0), wp, ldw, w2p,
-                                   _chk(out, "out", torch.bfloat16, 2), out.stride(0), st, ln, n_seg, N, K,
-                                   _EPI[epilogue], _chk(residual, "residual", torch.bfloat16, 2),
+                                   _chk(out, "out", odt, 2), out.stride(0), st, ln, n_seg, N, K,
+                                   epi, _chk(residual, "residual", odt, 2),
                                    residual.stride(0) if residual is not None else 0, gp,
                                    _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols),
                                    int(head_dim), _stream())
@@ -249,9 +268,10 @@ def grouped_gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wqs: Sequence[torch.Ten
     I64 = C.c_int64 * n_seg
     st, ln = I64(*[int(s) for s, _ in segments]), I64(*[int(l) for _, l in segments])
     half = head_dim // 2 if head_dim else 0
+    epi, odt = _epilogue(epilogue, out, residual)
     rc = lib.cdm_grouped_gemm_fp8(_chk(aq, "aq", FP8_DTYPE, 2), aq.stride(0), _f32vec(sa, "sa", M), wp, swp, ldw, w2p, sw2p,
-                                  _chk(out, "out", torch.bfloat16, 2), out.stride(0), st, ln, n_seg, N, K,
-                                  _EPI[epilogue], _chk(residual, "residual", torch.bfloat16, 2),
+                                  _chk(out, "out", odt, 2), out.stride(0), st, ln, n_seg, N, K,
+                                  epi, _chk(residual, "residual", odt, 2),
                                   residual.stride(0) if residual is not None else 0, gp,
                                   _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols),
                                   int(head_dim), _stream())

@@ -34,8 +34,9 @@ def axis_map(head_dim: int, sections: Sequence[int], layout: str = "chunked") ->
     return out
 
 
-def build_positions(n_text: int, grid: Sequence[int], n_action: int = 0) -> Tuple[torch.Tensor, List[Tuple[str, int, int]]]:
-    """Positions [3, N] of the joint sequence text | video | action, plus the (kind, start, length) runs.
+def build_positions(n_text: int, grid: Sequence[int], n_action: int = 0,
+                    n_audio: int = 0) -> Tuple[torch.Tensor, List[Tuple[str, int, int]]]:
+    """Positions [3, N] of the joint sequence text | video | audio | action, plus the (kind, start, length) runs.
 
     A 1-D run at offset s gets (s+j, s+j, s+j) and advances s by its length; a T x H x W grid gets
     (s+t, s+h, s+w) in row-major order and advances s by max(H, W).
@@ -52,10 +53,11 @@ def build_positions(n_text: int, grid: Sequence[int], n_action: int = 0) -> Tupl
         w = (torch.arange(W) + cur).view(1, 1, W).expand(T, H, W)
         pos.append(torch.stack([t.reshape(-1), h.reshape(-1), w.reshape(-1)]))
         runs.append(("video", tok, T * H * W)); tok += T * H * W; cur += max(H, W)
-    if n_action:
-        p = torch.arange(n_action, dtype=torch.long) + cur
-        pos.append(torch.stack([p, p, p]))
-        runs.append(("action", tok, n_action)); tok += n_action; cur += n_action
+    for kind, n in (("audio", n_audio), ("action", n_action)):      # 1-D runs like text
+        if n:
+            p = torch.arange(n, dtype=torch.long) + cur
+            pos.append(torch.stack([p, p, p]))
+            runs.append((kind, tok, n)); tok += n; cur += n
     return torch.cat(pos, dim=1), runs
 
 

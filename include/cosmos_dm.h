@@ -43,8 +43,10 @@ typedef enum cdm_epilogue {
     CDM_EPI_NONE = 0,          /* C = A W^T                                              */
     CDM_EPI_SWIGLU = 1,        /* C = silu(A Wg^T) * (A Wu^T)          (W = Wg, W2 = Wu) */
     CDM_EPI_GATE_RESIDUAL = 2, /* C = R + gate[n] * (A W^T)            (gate may be null = 1) */
-    CDM_EPI_ROPE_QK = 3        /* C = A W^T with rotate-half RoPE applied to the columns
+    CDM_EPI_ROPE_QK = 3,       /* C = A W^T with rotate-half RoPE applied to the columns
                                   below `rope_cols` (heads of width head_dim)            */
+    CDM_EPI_GATE_RESIDUAL_F32 = 4 /* CDM_EPI_GATE_RESIDUAL with C and R stored as fp32: the residual stream kept in
+                                  fp32 (28 roundings of the stream to bf16 alone cost percent-level accuracy) */
 } cdm_epilogue;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -71,6 +73,10 @@ int32_t cdm_device_count(void);
 int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const float* shift, const float* scale,
                                void* y, int64_t n_tokens, int64_t d, float eps, void* stream);
 
+/* The same operator reading an fp32 residual stream: x [n_tokens, d] fp32, y bf16 (the GEMM operand). */
+int32_t cdm_adaln_rmsnorm_f32(const float* x, const void* w, const float* shift, const float* scale,
+                              void* y, int64_t n_tokens, int64_t d, float eps, void* stream);
+
 /*
  * Same norm with a per-token e4m3 quantisation epilogue (fp8 variant of the block):
  *   s_tok[i] = max_j |y[i,j]| / 448 (0 -> 1);  yq[i,j] = e4m3(y[i,j] / s_tok[i])
@@ -79,6 +85,9 @@ int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const float* shift,
 int32_t cdm_adaln_rmsnorm_quant_e4m3(const void* x, const void* w, const float* shift, const float* scale,
                                      void* yq, float* s_tok, int64_t n_tokens, int64_t d, float eps,
                                      void* stream);
+int32_t cdm_adaln_rmsnorm_f32_quant_e4m3(const float* x, const void* w, const float* shift, const float* scale,
+                                         void* yq, float* s_tok, int64_t n_tokens, int64_t d, float eps,
+                                         void* stream);      /* x fp32 */
 
 /*
  * Per-row dynamic e4m3 quantisation of a bf16 matrix (activations before a quantised linear):
@@ -97,6 +106,7 @@ int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, float* s, int64
  *   fp32 accumulation on MFMA, one rounding to bf16 at the end.
  *   CDM_EPI_SWIGLU:        W = gate_proj.weight, W2 = up_proj.weight (same shape/ld), C: [M, N]
  *   CDM_EPI_GATE_RESIDUAL: R: [M, N] (ldr) residual (may alias C), gate: [N] fp32 or null
+ *   CDM_EPI_GATE_RESIDUAL_F32: the same with C and R fp32 (ldc, ldr in fp32 elements)
  *   CDM_EPI_ROPE_QK:       cos, sin: [M, head_dim/2] fp32; columns [0, rope_cols) are rotated
  *                          per head (pairs (i, i + head_dim/2)); head_dim in {64, 128};
  *                          rope_cols % 256 == 0

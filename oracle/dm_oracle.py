@@ -1,8 +1,13 @@
 """fp32 PyTorch restatement of the Cosmos 3 generator (DM) block forward.
 
 Test infrastructure: see the package docstring for who may import this and
-for the pinning status of every function.  Everything runs on the CPU in
-fp32 (statistics, softmax and accumulation included) and never rounds to bf16.
+for the pinning status of every function.  Everything is fp32 (statistics,
+softmax and accumulation included) and never rounds to bf16.  The functions
+allocate on the device of their inputs: the pinning tests and the parity tests
+run them on the CPU; for free-running checks of a whole stack at full size (hours
+on host cores) a GPU test may also hand them device tensors, which runs the very
+same statements through stock PyTorch fp32 operators (and checks that run
+against the CPU run on sampled rows first).
 
 Citations use ``REF/`` for the reference repository and ``TF/`` for the
 installed third-party ``transformers 5.15.0`` package, whose Cosmos 3 AR tower
@@ -133,15 +138,15 @@ def vision_positions(start: int, grid: Sequence[int]) -> torch.Tensor:
 
 
 def joint_positions(segments: Sequence[Tuple[str, object]]) -> torch.Tensor:
-    """Positions of a joint sequence of ("text", n) / ("video", (T,H,W)) / ("action", n) runs.
+    """Positions of a joint sequence of ("text", n) / ("video", (T,H,W)) / ("audio", n) / ("action", n) runs.
 
     Offsets advance by the run length after a 1-D run and by max(H, W) after a
-    grid (TF/models/cosmos3_omni/modeling_cosmos3_omni.py:241-259).  Action
-    tokens are a 1-D run like text (a choice; parity unpinned).
+    grid (TF/models/cosmos3_omni/modeling_cosmos3_omni.py:241-259).  Audio and
+    action tokens are 1-D runs like text (a choice; parity unpinned).
     """
     pos, cur = [], 0
     for kind, spec in segments:
-        if kind in ("text", "action"):
+        if kind in ("text", "audio", "action"):
             pos.append(text_positions(cur, int(spec)))
             cur += int(spec)
         elif kind == "video":
@@ -184,11 +189,11 @@ def apply_mrope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.
 # --------------------------------------------------------------------------
 # attention
 # --------------------------------------------------------------------------
-def hybrid_kv_end(n_tokens: int, causal_prefix: int) -> torch.Tensor:
+def hybrid_kv_end(n_tokens: int, causal_prefix: int, device=None) -> torch.Tensor:
     """Per-query key limit of the hybrid mask (architecture figure, right panel; REF/README.md:74): the first
     ``causal_prefix`` tokens (the AR / text run) see keys 0..i (causal, and no generator keys), all later tokens
     (DM, full attention) see every key.  Query i sees key j iff j < kv_end[i]."""
-    i = torch.arange(n_tokens)
+    i = torch.arange(n_tokens, device=device)
     return torch.where(i < causal_prefix, i + 1, torch.full_like(i, n_tokens))
 
 
@@ -208,7 +213,7 @@ def attention_rows(q_rows: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     kk, vv = _kv_heads(k, q.shape[0]), _kv_heads(v, q.shape[0])   # [H,N,dh]
     s = torch.matmul(q, kk.transpose(1, 2)) * (1.0 / math.sqrt(q.shape[-1]))
     if kv_end is not None:
-        hidden = torch.arange(k.shape[0]).view(1, 1, -1) >= kv_end.view(1, -1, 1)
+        hidden = torch.arange(k.shape[0], device=k.device).view(1, 1, -1) >= kv_end.view(1, -1, 1)
         s = s.masked_fill(hidden, float("-inf"))
     p = torch.softmax(s, dim=-1, dtype=torch.float32)
     return torch.matmul(p, vv).transpose(0, 1).contiguous()
@@ -234,7 +239,7 @@ def attention(q, k, v, chunk: int = 1024, kv_end: Optional[torch.Tensor] = None)
         qq = q[i:i + chunk].to(torch.float32).transpose(0, 1).contiguous()
         s = torch.matmul(qq, kk.transpose(1, 2)) * scale
         if kv_end is not None:
-            hidden = torch.arange(k.shape[0]).view(1, 1, -1) >= kv_end[i:i + chunk].view(1, -1, 1)
+            hidden = torch.arange(k.shape[0], device=k.device).view(1, 1, -1) >= kv_end[i:i + chunk].view(1, -1, 1)
             s = s.masked_fill(hidden, float("-inf"))
         p = torch.softmax(s, dim=-1, dtype=torch.float32)
         out.append(torch.matmul(p, vv).transpose(0, 1))
@@ -314,7 +319,8 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
         segments = [(0, N, 0, mod is not None)]
     dkv = weight_sets[segments[0][2]]["wk"].shape[0]
     n_kv = dkv // dh
-    q = torch.empty(N, d); k = torch.empty(N, dkv); v = torch.empty(N, dkv)
+    dev = x.device
+    q = torch.empty(N, d, device=dev); k = torch.empty(N, dkv, device=dev); v = torch.empty(N, dkv, device=dev)
     for (s0, ln, ws, modulated) in segments:
         p = weight_sets[ws]
         sl = slice(s0, s0 + ln)
@@ -327,12 +333,12 @@ def dm_block(x: torch.Tensor, weight_sets: Sequence[Dict[str, torch.Tensor]],
     q = apply_mrope(q.view(N, n_heads, dh), cos, sin)
     k = apply_mrope(k.view(N, n_kv, dh), cos, sin)
     v = v.view(N, n_kv, dh)
-    kv_end = hybrid_kv_end(N, causal_prefix) if causal_prefix else None
+    kv_end = hybrid_kv_end(N, causal_prefix, dev) if causal_prefix else None
     if attn_rows is None:
         o = attention(q, k, v, kv_end=kv_end).reshape(N, d)
-        rows = torch.arange(N)
+        rows = torch.arange(N, device=dev)
     else:
-        rows = attn_rows
+        rows = attn_rows.to(dev)
         o = attention_rows(q[rows], k, v, kv_end[rows] if kv_end is not None else None).reshape(-1, d)
     xr = x[rows]
     out = torch.empty_like(xr)

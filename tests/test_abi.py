@@ -27,7 +27,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} declared in include/cosmos_dm.h but not exported"
     assert set(names) == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
     assert lib.cdm_version() >= 100
-    assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 2 * 128 * 2 * 64 * 2
+    # two tile images of 128 padded tokens x 2 heads x 64 channels (bf16) + one fp32 key-norm bound per (head, tile)
+    assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 2 * 128 * 2 * 64 * 2 + 2 * 2 * 4
 
 
 def test_bad_arguments_are_rejected_on_the_host():

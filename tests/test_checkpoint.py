@@ -25,8 +25,11 @@ def test_attested_key_names_are_classified():
     assert classify("layers.1.post_attention_layernorm.weight") == (1, ("block", "norm2_weight"), AR)
     assert classify("proj_in.bias")[1] == ("top", "proj_in.bias")
     assert classify("time_embedder.linear_1.weight")[1][0] == "top"
-    # not part of the generator path: sound tower, embeddings, the vision encoder
-    for k in ("audio_proj_in.weight", "embed_tokens.weight", "blocks.0.attn.qkv.weight", "lm_head.weight"):
+    # the sound stream's edges are stack-level tensors like the action stream's
+    assert classify("audio_proj_in.weight")[1] == ("top", "audio_proj_in.weight")
+    assert classify("audio_modality_embed")[1] == ("top", "audio_modality_embed")
+    # not part of the generator path: embeddings, the vision encoder
+    for k in ("embed_tokens.weight", "blocks.0.attn.qkv.weight", "lm_head.weight", "audio_encoder.conv.weight"):
         assert classify(k) is None
 
 

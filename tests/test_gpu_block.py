@@ -518,3 +518,169 @@ def test_batched_forward_is_a_loop_over_samples():
     d = m.stack(torch.randn((2, cfg.n_video, 256), generator=g, device=dev()).to(torch.bfloat16), t, encoder_hidden_states=ctx,
                 action_states=torch.randn((2, 5, 256), generator=g, device=dev()).to(torch.bfloat16), return_dict=True)
     assert d["sample"].shape == (2, cfg.n_video, 256) and d["joint"].shape == (2, cfg.n_tokens, 256)
+
+
+class _RMSNorm(torch.nn.Module):
+    def __init__(self, dim, eps=1e-6):
+        super().__init__()
+        self.weight, self.eps = torch.nn.Parameter(torch.ones(dim)), eps
+
+
+class _JointAttention(torch.nn.Module):
+    """Stand-in for the attention module of the reference's transformer: nothing but the attested sub-module names
+    (to_q / to_k / to_v / to_out[0], add_q_proj / add_k_proj / add_v_proj / to_add_out, norm_q / norm_k /
+    norm_added_q / norm_added_k), a head count and the diffusers processor plumbing."""
+
+    def __init__(self, d, heads, kv_heads, qk_norm=True):
+        super().__init__()
+        L = lambda i, o: torch.nn.Linear(i, o, bias=False)
+        hd = d // heads
+        self.heads = heads
+        self.to_q, self.to_k, self.to_v = L(d, d), L(d, kv_heads * hd), L(d, kv_heads * hd)
+        self.to_out = torch.nn.ModuleList([L(d, d), torch.nn.Dropout(0.0)])
+        self.add_q_proj, self.add_k_proj, self.add_v_proj, self.to_add_out = L(d, d), L(d, kv_heads * hd), L(d, kv_heads * hd), L(d, d)
+        if qk_norm:
+            self.norm_q, self.norm_k, self.norm_added_q, self.norm_added_k = (_RMSNorm(hd) for _ in range(4))
+        self.processor = None
+
+    def set_processor(self, processor):
+        self.processor = processor
+
+    def forward(self, hidden_states, encoder_hidden_states=None, attention_mask=None, image_rotary_emb=None, **kw):
+        return self.processor(self, hidden_states, encoder_hidden_states=encoder_hidden_states,
+                              attention_mask=attention_mask, image_rotary_emb=image_rotary_emb, **kw)
+
+
+@pytest.mark.parametrize("kv_heads", [2, 1])
+def test_processor_drops_onto_a_diffusers_style_attention_module(kv_heads):
+    """attn.set_processor(DMAttnProcessor()) on a module that only carries the reference's sub-module names: the fused
+    QKV views are built once, the module's own weights become views of them (one copy of the weights), and the result
+    matches the oracle; a later change of the weights is picked up."""
+    from cosmos_amd import DMAttnProcessor
+    d, heads, hd, n_ctx, n_lat = 256, 2, 128, 16, 32
+    torch.manual_seed(3)
+    attn = _JointAttention(d, heads, kv_heads).to(dev()).to(torch.bfloat16)
+    with torch.no_grad():
+        for p in attn.parameters():
+            p.copy_(torch.randn_like(p.float()) * (0.06 if p.dim() == 2 else 0.3) + (0.0 if p.dim() == 2 else 1.0))
+    attn.set_processor(DMAttnProcessor())
+    n_bytes_before = sum(p.numel() * p.element_size() for p in attn.parameters())
+    g = torch.Generator().manual_seed(21)
+    h, hr = rand_bf16((1, n_lat, d), g)
+    e, er = rand_bf16((1, n_ctx, d), g)
+    pos, _ = rotary.build_positions(n_ctx, (1, 4, 8))
+    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48))
+    rot = (cos.to(dev()), sin.to(dev()))
+
+    def oracle():
+        f = lambda m: m.weight.detach().float().cpu()
+        x = torch.cat([er[0], hr[0]])
+        br = [(attn.to_q, attn.to_k, attn.to_v, attn.to_out[0], attn.norm_q, attn.norm_k),
+              (attn.add_q_proj, attn.add_k_proj, attn.add_v_proj, attn.to_add_out, attn.norm_added_q, attn.norm_added_k)]
+        sl = [slice(0, n_ctx), slice(n_ctx, n_ctx + n_lat)]
+        q = torch.cat([O.rms_norm((x[s] @ f(b[0]).t()).view(-1, heads, hd), f(b[4])).reshape(-1, d) for b, s in zip(br, sl)])
+        k = torch.cat([O.rms_norm((x[s] @ f(b[1]).t()).view(-1, kv_heads, hd), f(b[5])).reshape(-1, kv_heads * hd) for b, s in zip(br, sl)])
+        v = torch.cat([x[s] @ f(b[2]).t() for b, s in zip(br, sl)])
+        n = n_ctx + n_lat
+        o = O.attention(O.apply_mrope(q.view(n, heads, hd), cos, sin), O.apply_mrope(k.view(n, kv_heads, hd), cos, sin),
+                        v.view(n, kv_heads, hd)).reshape(n, d)
+        return o[n_ctx:] @ f(attn.to_add_out).t(), o[:n_ctx] @ f(attn.to_out[0]).t()
+
+    ho, eo = attn(h, encoder_hidden_states=e, image_rotary_emb=rot)
+    assert ho.shape == (1, n_lat, d) and eo.shape == (1, n_ctx, d)
+    want_h, want_e = oracle()
+    assert_close(ho[0], want_h, BF16_COS, BF16_REL, "adopted module: latent stream")
+    assert_close(eo[0], want_e, BF16_COS, BF16_REL, "adopted module: context stream")
+    # one copy of the weights: q / k / v of a branch are consecutive row ranges of one fused tensor
+    dkv = kv_heads * hd
+    assert attn.to_k.weight.data_ptr() == attn.to_q.weight.data_ptr() + d * d * 2
+    assert attn.add_v_proj.weight.data_ptr() == attn.add_q_proj.weight.data_ptr() + (d + dkv) * d * 2
+    assert sum(p.numel() * p.element_size() for p in attn.parameters()) == n_bytes_before
+    assert "_cdm_adopted" not in dict(attn.named_modules()) and all("cdm" not in k for k in attn.state_dict())
+    adopted = attn.__dict__["_cdm_adopted"]
+    ho2, _ = attn(h, encoder_hidden_states=e, image_rotary_emb=rot)
+    assert attn.__dict__["_cdm_adopted"] is adopted and torch.equal(ho, ho2)          # built once
+    # load_state_dict writes through the views; a replaced norm weight is noticed
+    sd = {k: (v.float() * 1.5).to(v.dtype) if k.startswith("add_v_proj") else v.clone() for k, v in attn.state_dict().items()}
+    attn.load_state_dict(sd)
+    with torch.no_grad():
+        attn.norm_added_q.weight.mul_(0.5)
+    ho3, eo3 = attn(h, encoder_hidden_states=e, image_rotary_emb=rot)
+    want_h3, want_e3 = oracle()
+    assert O.max_rel_err(want_h3, want_h) > 5e-2
+    assert_close(ho3[0], want_h3, BF16_COS, BF16_REL, "adopted module after a weight update: latent stream")
+    assert_close(eo3[0], want_e3, BF16_COS, BF16_REL, "adopted module after a weight update: context stream")
+    with pytest.raises(NotImplementedError):
+        attn(h, attention_mask=torch.ones(1, n_lat, device=dev()), image_rotary_emb=rot)
+
+
+def test_four_modality_block_with_audio():
+    """text | video | audio | action with four weight sets (and with audio on the generator's set when there are only
+    three): the block against the fp32 oracle (which the CPU suite pins to the float64 brute force on this layout)."""
+    for nb in (4, 3):
+        cfg = DMConfig("av", 256, 2, 128, 512, 1, (2, 4, 8), n_text=40, n_action=24, n_audio=19, n_branches=nb)
+        st = DMStack(cfg, device=dev())
+        blk = make_block(cfg, 61 + nb)
+        g = torch.Generator().manual_seed(61)
+        x, xr = rand_bf16((cfg.n_tokens, 256), g)
+        temb, tembr = rand_bf16((256,), g)
+        segs = st.segments()
+        audio_branch = 3 if nb == 4 else 1
+        assert segs == [(0, 40, 0, False), (40, 64, 1, True), (104, 19, audio_branch, True), (123, 24, 2, True)]
+        y = blk(x, temb, st.rotary(dev()), segs)
+        mod = O.adaln_modulation(tembr.view(1, -1), blk.adaLN_modulation.weight.float().cpu(),
+                                 blk.adaLN_modulation.bias.float().cpu())
+        pos = O.joint_positions([("text", 40), ("video", cfg.grid), ("audio", 19), ("action", 24)])
+        assert torch.equal(pos, rotary.build_positions(40, cfg.grid, 24, 19)[0])
+        # audio positions continue after the grid's offset max(H, W) and action positions after the audio run
+        assert int(pos[0, 104]) == 40 + 8 and int(pos[0, 123]) == 40 + 8 + 19
+        cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+        want = O.dm_block(xr, oracle_weights(blk, nb), mod, cos, sin, 2, segs)
+        assert_close(y, want, BF16_COS, BF16_REL, f"four-modality block, {nb} weight sets")
+
+
+def test_transformer_with_audio_stream_and_context_cache():
+    """DMTransformer with sound and action streams: outputs per stream; under the hybrid mask the cached text K/V
+    (context_cache) give the same prediction as the joint forward."""
+    from cosmos_amd import DMTransformer
+    cfg = DMConfig("snd", 256, 2, 128, 512, 2, (2, 3, 4), n_text=64, n_action=5, n_audio=9, n_branches=4, qk_norm=True,
+                   hybrid_mask=True)
+    m = DMTransformer(cfg, latent_channels=4, action_dim=6, audio_dim=10, device=dev())
+    m.reset_parameters(5)
+    g = torch.Generator(device=dev()).manual_seed(5)
+    with torch.no_grad():
+        m.audio_modality_embed.copy_(0.5 * torch.randn(256, generator=g, device=dev()))
+        for blk in m.stack.blocks:
+            blk.adaLN_modulation.bias.copy_(0.3 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
+    assert {"audio_proj_in.weight", "audio_proj_out.bias", "audio_modality_embed"} <= set(m.top_level_keys())
+    lat = torch.randn((1, 4, 2, 6, 8), generator=g, device=dev())
+    ctx = torch.randn((1, 64, 256), generator=g, device=dev()).to(torch.bfloat16)
+    act = torch.randn((1, 5, 6), generator=g, device=dev())
+    snd = torch.randn((1, 9, 10), generator=g, device=dev())
+    t = torch.tensor([450.0], device=dev())
+    out = m(lat, t, encoder_hidden_states=ctx, action_states=act, audio_states=snd, return_dict=True)
+    assert out["sample"].shape == lat.shape and out["audio"].shape == (1, 9, 10) and out["action"].shape == (1, 5, 6)
+    tup = m(lat, t, encoder_hidden_states=ctx, action_states=act, audio_states=snd)
+    assert len(tup) == 3 and torch.equal(tup[1], out["audio"]) and torch.equal(tup[2], out["action"])
+    with pytest.raises(ValueError):
+        m(lat, t, encoder_hidden_states=ctx, action_states=act)
+    cache = m.stack.precompute_context(ctx)
+    out2 = m(lat, t, action_states=act, audio_states=snd, return_dict=True, context_cache=cache)
+    for k in ("sample", "audio", "action"):
+        assert_close(out2[k], out[k].float().cpu(), 0.9999, 1e-2, f"transformer with context cache: {k}")
+    # oracle: audio rows of the stack
+    f = lambda p: p.detach().float().cpu()
+    tok = m.patchify(lat[0].to(torch.bfloat16)).float().cpu() @ f(m.proj_in.weight).t() + f(m.proj_in.bias)
+    a_in = f(act[0].to(torch.bfloat16)) @ f(m.action_proj_in.weight).t() + f(m.action_proj_in.bias) + f(m.action_modality_embed)
+    s_in = f(snd[0].to(torch.bfloat16)) @ f(m.audio_proj_in.weight).t() + f(m.audio_proj_in.bias) + f(m.audio_modality_embed)
+    x = torch.cat([f(ctx[0]), tok, s_in, a_in])
+    te = m.time_embedder
+    c = O.time_mlp(O.timestep_embedding(t.cpu()), f(te.linear_1.weight), f(te.linear_1.bias), f(te.linear_2.weight), f(te.linear_2.bias))
+    mods = [O.adaln_modulation(c, f(b.adaLN_modulation.weight), f(b.adaLN_modulation.bias)) for b in m.stack.blocks]
+    pos = O.joint_positions([("text", 64), ("video", cfg.grid), ("audio", 9), ("action", 5)])
+    cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
+    y = O.dm_stack(x, [oracle_weights(b, 4) for b in m.stack.blocks], mods, cos, sin, 2, m.stack.segments(), causal_prefix=64)
+    y = O.rms_norm(y, f(m.norm_out), cfg.eps)
+    n0 = 64 + cfg.n_video
+    assert_close(out["audio"][0], y[n0:n0 + 9] @ f(m.audio_proj_out.weight).t() + f(m.audio_proj_out.bias), BF16_COS, BF16_REL, "audio head")
+    assert_close(out["action"][0], y[n0 + 9:] @ f(m.action_proj_out.weight).t() + f(m.action_proj_out.bias), BF16_COS, BF16_REL, "action head (after audio)")

@@ -33,6 +33,26 @@ def test_adaln_rmsnorm(n, d, modulated):
     assert torch.equal(y2, y)
 
 
+@pytest.mark.parametrize("n,d", [(37, 1024), (300, 4096), (5, 8192), (9, 1160)])
+def test_adaln_rmsnorm_fp32_stream(n, d):
+    """The same norm reading a residual stream kept in fp32 (bf16 out, and the e4m3 + per-token-scale form)."""
+    g = gen(n * 11 + d)
+    xr = torch.randn((n, d), generator=g) * 2.0
+    w, wr = rand_bf16((d,), g)
+    sh, sc = torch.randn(d, generator=g), torch.randn(d, generator=g) * 0.5
+    y = ops.adaln_rmsnorm(xr.to(dev()), w, sh.to(dev()), sc.to(dev()), 1e-6)
+    assert y.dtype == torch.bfloat16
+    want = O.adaln_rms_norm(xr, wr, sh, sc, 1e-6)
+    assert_close(y, want, 0.99999, 6e-3, f"adaln_rmsnorm fp32 in {n}x{d}")
+    # a bf16-representable input gives the bits of the bf16-input kernel
+    xb = xr.to(torch.bfloat16)
+    assert torch.equal(ops.adaln_rmsnorm(xb.float().to(dev()), w, sh.to(dev()), sc.to(dev()), 1e-6),
+                       ops.adaln_rmsnorm(xb.to(dev()), w, sh.to(dev()), sc.to(dev()), 1e-6))
+    q1, s1 = ops.adaln_rmsnorm_quant(xb.float().to(dev()), w, sh.to(dev()), sc.to(dev()), 1e-6)
+    q2, s2 = ops.adaln_rmsnorm_quant(xb.to(dev()), w, sh.to(dev()), sc.to(dev()), 1e-6)
+    assert torch.equal(q1.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s1, s2)
+
+
 def test_adaln_rmsnorm_closed_form():
     d = 512
     x = torch.full((3, d), 2.5, dtype=torch.bfloat16, device=dev())
@@ -197,6 +217,40 @@ def test_grouped_gemm_fp8_and_gaps(variant, request):
     assert torch.equal(out, ref)
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("M,N,K,gated,fp8", [(256, 256, 128, True, False), (300, 1024, 512, True, False), (77, 264, 128, False, False),
+                                             (515, 520, 256, True, True), (1030, 4096, 1024, True, False)])
+def test_gemm_gate_residual_fp32_stream(M, N, K, gated, fp8, variant, request):
+    """Gated residual with the residual stream (R and C, in place) kept in fp32: one rounding less per block."""
+    prev = ops.set_variant("gemm", variant)
+    request.addfinalizer(lambda: ops.set_variant("gemm", prev))
+    g = gen(M + N + K + 5)
+    a, ar = rand_bf16((M, K), g)
+    w, wr = rand_bf16((N, K), g, 0.05)
+    rr = torch.randn((M, N), generator=g)
+    gate = torch.randn(N, generator=g) if gated else None
+    res = rr.to(dev())
+    if fp8:
+        aq, sa = ops.quant_rows(a); wq, sw = ops.quant_rows(w)
+        out = ops.gemm_fp8(aq, sa, wq, sw, epilogue="gate_residual", residual=res, gate=gate.to(dev()) if gated else None, out=res)
+        prod = O.fp8_linear(ar, wr)
+    else:
+        out = ops.gemm(a, w, epilogue="gate_residual", residual=res, gate=gate.to(dev()) if gated else None, out=res)
+        prod = ar @ wr.t()
+    assert out.dtype == torch.float32 and out.data_ptr() == res.data_ptr()
+    want = rr + (gate * prod if gated else prod)
+    assert_close(out, want, 0.99999, 2e-3 if not fp8 else 5e-3, f"gate_residual fp32 stream {M}x{N}x{K}")
+    if not fp8:
+        # against the bf16-stream epilogue on a bf16-representable residual: equal up to that epilogue's final rounding
+        rb = rr.to(torch.bfloat16)
+        o16 = ops.gemm(a, w, epilogue="gate_residual", residual=rb.to(dev()), gate=gate.to(dev()) if gated else None)
+        o32 = ops.gemm(a, w, epilogue="gate_residual", residual=rb.float().to(dev()), gate=gate.to(dev()) if gated else None,
+                       out=torch.empty((M, N), dtype=torch.float32, device=dev()))
+        assert torch.equal(o32.to(torch.bfloat16), o16)
+    with pytest.raises(TypeError):
+        ops.gemm(a, w, epilogue="gate_residual", residual=rr.to(torch.bfloat16).to(dev()), out=torch.empty((M, N), dtype=torch.float32, device=dev()))
+
+
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("n,H,hd", [(64, 2, 64), (256, 1, 128), (1000, 3, 128), (321, 2, 64), (1, 1, 128), (130, 2, 128), (65, 1, 64),
@@ -338,6 +392,62 @@ def test_attention_with_prefix_key_images(P, m, H, hd):
                     O.rms_norm(qkvr[P:, d:2 * d].view(m, H, hd), kw[1], 1e-6)])
     want = O.attention(O.apply_mrope(qn, cos[P:], sin[P:]), O.apply_mrope(kn, cos, sin), qkvr[:, 2 * d:].view(n, H, hd))
     assert_close(o, want.reshape(m, d), 0.9999, 1e-2, f"prefix images P={P} m={m}")
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n,hd", [(100, 64), (200, 128), (70, 128), (64, 64)])
+def test_attention_with_strongly_negative_logits(n, hd, variant, request):
+    """Every score of every row far below zero (about -170 in log2 units) and a ragged last tile: the zero keys
+    that pad the tile must never be taken for the row maximum (that would scale the sums towards zero)."""
+    prev = ops.set_variant("attn", variant)
+    request.addfinalizer(lambda: ops.set_variant("attn", prev))
+    g = gen(n + hd)
+    u = torch.ones(hd)
+    c = (120.0 * math.sqrt(hd) / hd) ** 0.5       # q.k / sqrt(hd) = -c^2 hd / sqrt(hd) = -120 (natural units)
+    kr = (c * u + 0.05 * torch.randn(n, hd, generator=g)).to(torch.bfloat16)
+    qr = (-c * u + 0.05 * torch.randn(n, hd, generator=g)).to(torch.bfloat16)
+    vr = torch.randn(n, hd, generator=g).to(torch.bfloat16)
+    o = ops.attention(qr.to(dev()), kr.to(dev()), vr.to(dev()), 1, hd)
+    want = O.attention(qr.float().view(n, 1, hd), kr.float().view(n, 1, hd), vr.float().view(n, 1, hd)).reshape(n, hd)
+    assert float((qr.float() @ kr.float().t()).max()) / math.sqrt(hd) < -100.0
+    assert_close(o, want, 0.9999, 1e-2, f"attention with strongly negative logits n={n}")
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("case", ["large_norms", "late_spike", "spike_in_first_tile", "tiny_norms"])
+def test_attention_reference_handling(case, variant, request):
+    """The default kernel bounds every score of a row by |q| max|k| and, where that bound stays within 2^60 of the first
+    tile's row maximum, runs without row maxima and reference updates; otherwise (and always in variants 1 and 2) the
+    running reference follows the row maxima.  large_norms: the bound is far too loose (safe loop) while the scores
+    are moderate; late_spike: one key far down the sequence beats everything before it by more than 2^60 for some
+    rows (the reference has to move, a lot); spike_in_first_tile: the reverse; tiny_norms: the fast loop."""
+    prev = ops.set_variant("attn", variant)
+    request.addfinalizer(lambda: ops.set_variant("attn", prev))
+    n, H, hd = 700, 2, 128
+    g = gen(len(case) * 3 + 1)
+    q = torch.randn(n, H, hd, generator=g)
+    k = torch.randn(n, H, hd, generator=g)
+    v = torch.randn(n, H, hd, generator=g)
+    if case == "large_norms":
+        q, k = q * 6.0, k * 6.0
+    elif case == "tiny_norms":
+        q, k = q * 0.05, k * 0.05
+    else:
+        at = 650 if case == "late_spike" else 7
+        k[at] = 9.0 * q[::2].mean(0) / q[::2].mean(0).norm(dim=-1, keepdim=True) * math.sqrt(hd)   # aligned with half of the queries
+        q = q * 3.0
+    qb, kb, vb = (t.to(torch.bfloat16) for t in (q, k, v))
+    o = ops.attention(qb.reshape(n, H * hd).to(dev()), kb.reshape(n, H * hd).to(dev()), vb.reshape(n, H * hd).to(dev()), H, hd)
+    want = O.attention(qb.float(), kb.float(), vb.float()).reshape(n, H * hd)
+    if case in ("late_spike", "spike_in_first_tile"):
+        s = torch.einsum("nhd,mhd->hnm", qb.float(), kb.float()) / math.sqrt(hd) * 1.4427
+        other = torch.cat([s[:, :, :at], s[:, :, at + 1:]], dim=2).amax(-1)
+        assert float((s[:, :, at] - other).amax()) > 70.0          # some rows are dominated by more than 2^60
+    # the kernels multiply Q by log2(e)/sqrt(hd) ahead of its one rounding to bf16, so a score carries a relative error of
+    # about 2^-9: invisible at ordinary logits, percent-level in the probabilities where logits of 50 - 150 (log2 units)
+    # compete, as they do here.  All variants share it; what this test is after is the handling of the reference.
+    loose = case != "tiny_norms"
+    assert_close(o, want, 0.9999, 8e-2 if loose else 1e-2, f"attention reference handling: {case} variant={variant}")
 
 
 def test_attention_closed_forms_and_determinism():

@@ -63,6 +63,28 @@ def test_block_vs_brute_mot_three_segments():
     assert torch.allclose(yr, y[rows], atol=1e-5)
 
 
+def test_block_vs_brute_four_modalities_with_audio():
+    """text | video | audio | action, four weight sets: audio is a 1-D run after the video grid (offset max(H, W)),
+    action follows it."""
+    g = torch.Generator().manual_seed(4)
+    d, H, h = 16, 2, 24
+    pos = O.joint_positions([("text", 4), ("video", (1, 2, 3)), ("audio", 3), ("action", 2)])
+    assert pos[:, 10:13].tolist() == [[7, 8, 9]] * 3 and pos[:, 13:].tolist() == [[10, 11]] * 3      # 4 + max(2, 3) = 7
+    N = pos.shape[1]
+    segments = [(0, 4, 0, False), (4, 6, 1, True), (10, 3, 3, True), (13, 2, 2, True)]
+    ws = [_weights(g, d, h) for _ in range(4)]
+    x = torch.randn(N, d, generator=g)
+    mod = [torch.randn(d, generator=g) * 0.5 for _ in range(6)]
+    cos, sin = O.mrope_cos_sin(pos, d // H, (4, 2, 2), 10000.0, "chunked")
+    y = O.dm_block(x, ws, mod, cos, sin, H, segments)
+    amap = O.mrope_axis_map(d // H, (4, 2, 2)).numpy()
+    yb = B.dm_block(x.numpy(), [_np(w) for w in ws], [m.double().numpy() for m in mod], pos.numpy(), amap, H, segments)
+    assert np.abs(y.numpy() - yb).max() < 2e-4 * np.abs(yb).max()
+    # the audio run really uses its own weights
+    ws2 = ws[:3] + [ws[1]]
+    assert float((O.dm_block(x, ws2, mod, cos, sin, H, segments) - y)[10:13].abs().max()) > 1e-3
+
+
 def test_rms_norm_closed_forms():
     d = 32
     w = torch.linspace(0.5, 1.5, d); sc = torch.linspace(-0.2, 0.3, d); sh = torch.linspace(-1, 1, d)
