@@ -28,13 +28,14 @@ ATTN_TRAFFIC_BYTES = {(56832, 32, 128): 8.61e9 + 0.466e9}
 
 
 def cpu_baseline(cfg, sample_tokens: int):
-    """fp32 oracle of ONE block on `sample_tokens` tokens of the same width, timed on the host cores; the GEMM
-    part scales linearly and the attention part quadratically with the token count."""
+    """fp32 oracle of ONE block on `sample_tokens` tokens of the same width (0 = all tokens: minutes of CPU time at the
+    benchmark sizes), timed on the host cores; the GEMM part scales linearly and the attention part quadratically with
+    the token count."""
     import torch
     import oracle as O
     d, h, H = cfg.d_model, cfg.hidden, cfg.n_heads
     g = torch.Generator().manual_seed(0)
-    n = sample_tokens
+    n = min(sample_tokens, cfg.n_tokens) if sample_tokens > 0 else cfg.n_tokens
     x = torch.randn(n, d, generator=g)
     w = dict(norm1_w=torch.ones(d), norm2_w=torch.ones(d))
     for name, shape in (("wq", (d, d)), ("wk", (d, d)), ("wv", (d, d)), ("wo", (d, d)), ("wg", (h, d)), ("wu", (h, d)),
@@ -56,7 +57,8 @@ def cpu_baseline(cfg, sample_tokens: int):
     t_lin = max(t_block - t_attn, 0.0)
     ratio = cfg.n_tokens / n
     per_block = t_lin * ratio + t_attn * ratio * ratio
-    return {"value": round(per_block * max(cfg.n_blocks, 1) * 1e3, 1), "unit": "ms per denoising step (extrapolated)",
+    return {"value": round(per_block * max(cfg.n_blocks, 1) * 1e3, 1),
+            "unit": "ms per denoising step (extrapolated)" if (ratio > 1 or cfg.n_blocks > 1) else "ms per denoising step",
             "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"fp32 oracle, one block on {n} of {cfg.n_tokens} tokens at full width: {t_block:.2f} s "
                       f"(attention {t_attn:.2f} s); linear part x{ratio:.2f}, attention x{ratio * ratio:.1f}, "
@@ -113,6 +115,8 @@ def main():
     ap.add_argument("--attn-variant", type=int, default=0)
     ap.add_argument("--gemm-variant", type=int, default=0)
     ap.add_argument("--rope", default="in_attention", choices=["in_attention", "gemm_epilogue", "streaming"])
+    ap.add_argument("--graph", action="store_true",
+                    help="record the forward into a HIP graph once and time replays (launch-bound shapes such as C0)")
     ap.add_argument("--residual", default="fp32", choices=["fp32", "bf16"],
                     help="dtype the residual stream is kept in between blocks (fp32 = the default of a stack)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
@@ -152,14 +156,22 @@ def main():
         from cosmos_amd import DMAttnProcessor
         for blk in stack.blocks:
             blk.attn.set_processor(DMAttnProcessor(rope=args.rope))
-    g = torch.Generator(device=dev).manual_seed(cfg.seed)
+    # the weights were drawn from a generator seeded with cfg.seed: the inputs take another stream (the same seed would
+    # reproduce the weights' random numbers, i.e. token rows parallel to weight rows)
+    g = torch.Generator(device=dev).manual_seed(cfg.seed + 1000)
     xv = torch.randn((1, cfg.n_video, cfg.d_model), generator=g, device=dev).to(torch.bfloat16)
     xt = torch.randn((1, cfg.n_text, cfg.d_model), generator=g, device=dev).to(torch.bfloat16) if cfg.n_text else None
     xa = torch.randn((1, cfg.n_action, cfg.d_model), generator=g, device=dev).to(torch.bfloat16) if cfg.n_action else None
     t = torch.rand(1, generator=g, device=dev) * 1000.0
 
-    def step():
-        return stack(xv, t, encoder_hidden_states=xt, action_states=xa)[0]
+    if args.graph:
+        graphed = stack.capture(xv, t, encoder_hidden_states=xt, action_states=xa)
+
+        def step():
+            return graphed(xv, t, encoder_hidden_states=xt, action_states=xa)["sample"]
+    else:
+        def step():
+            return stack(xv, t, encoder_hidden_states=xt, action_states=xa)[0]
 
     for _ in range(args.warmup):
         step()
@@ -184,7 +196,8 @@ def main():
 
     ms_per_step = wall * 1e3 / args.steps
     attn_ms = [a.elapsed_time(b) for a, b in events]
-    if not attn_ms:      # measurement variants of the attention kernel are timed as a whole by rocprof only
+    timed_launches = len(attn_ms)
+    if not attn_ms:      # graph replays launch nothing from Python: no per-launch events; figures below are then null
         attn_ms = [float("nan")]
     attn_avg_ms = sum(attn_ms) / len(attn_ms)
     attn_flops = cfg.attn_flops_per_block()
@@ -221,11 +234,13 @@ def main():
                                f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
                    "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope,
-                   "residual_stream": args.residual},
+                   "residual_stream": args.residual, "hip_graph": bool(args.graph)},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4),
                      "traffic": ATTN_TRAFFIC_BYTES.get((cfg.n_tokens, cfg.n_heads, cfg.head_dim))
                      if args.attn_variant == 0 else None,
+                     "traffic_source": "stored figure of two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) over this kernel at "
+                                       "this shape, profiles/c2_one_block_pmc_counters.txt; counters cannot be read in-process",
                      "flops_per_launch": attn_flops, "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms)},
         "kernels": kernels,
         "extra": {"ms_per_block": round(ms_per_step / cfg.n_blocks, 3),
@@ -237,7 +252,12 @@ def main():
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
-    print(json.dumps(res))
+    def no_nan(o):
+        if isinstance(o, dict):
+            return {k: no_nan(v) for k, v in o.items()}
+        return None if isinstance(o, float) and o != o else o
+    res["roofline"]["launches"] = timed_launches
+    print(json.dumps(no_nan(res)))
 
 
 if __name__ == "__main__":

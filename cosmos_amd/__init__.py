@@ -7,7 +7,7 @@ from . import _lib, ops, rotary  # noqa: F401
 from .config import DMConfig, CONFIGS  # noqa: F401
 from .sampler import FlowEulerStepper, UniPCStepper, flow_sigmas  # noqa: F401
 from .modules import (AdoptedAttention, DMAttention, DMAttnProcessor, DMBlock, DMStack, DMTransformer,  # noqa: F401
-                      TimestepEmbedder, Workspace, adopt_attention)
+                      GraphedStack, TimestepEmbedder, Workspace, adopt_attention)
 from .checkpoint import export_generator_weights, load_generator_weights  # noqa: F401
 
 __version__ = "0.1.0"

@@ -200,8 +200,13 @@ class _AttentionCore:
         ends = [s0 + ln for (s0, ln, _, _) in segments]
         qw, kw = _data(self.norm_q_weight), _data(self.norm_k_weight)
         if branches != list(range(self.n_branches)):
-            idx = torch.tensor(branches, device=qw.device)
-            qw, kw = qw.index_select(0, idx).contiguous(), kw.index_select(0, idx).contiguous()
+            # the index tensor is made once per segment layout: a later call may run under graph capture, where a
+            # host-to-device copy is not allowed
+            cache = self.__dict__.setdefault("_branch_idx", {})
+            key = (tuple(branches), str(qw.device))
+            if key not in cache:
+                cache[key] = torch.tensor(branches, device=qw.device)
+            qw, kw = qw.index_select(0, cache[key]).contiguous(), kw.index_select(0, cache[key]).contiguous()
         return qw, kw, ends, self.qk_eps
 
     def _linear(self, a: torch.Tensor, sa: Optional[torch.Tensor], which: str, segments: Sequence[Segment], *,
@@ -601,6 +606,17 @@ class DMStack(nn.Module):
             blk(x, temb, rot, segs, inplace=True, workspace=self._ws, causal_prefix=c.n_text if c.hybrid_mask else 0)
         return self._result(x, c.n_text, hidden_states.dim() == 3, return_dict)
 
+    def capture(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
+                encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
+                audio_states: Optional[torch.Tensor] = None, context_cache: Optional["ContextCache"] = None) -> "GraphedStack":
+        """Record one forward (batch 1) on inputs of these shapes into a HIP graph and return the replayer: for
+        launch-bound shapes (a few thousand tokens at small width: a dozen launches per block of microseconds each) a
+        replay costs one launch instead of a dozen per block.  The kernels take every size from host arguments at
+        capture time, so a graph serves exactly the shapes it was recorded with."""
+        return GraphedStack(self, dict(hidden_states=hidden_states, timestep=timestep,
+                                       encoder_hidden_states=encoder_hidden_states, action_states=action_states,
+                                       audio_states=audio_states), context_cache)
+
     def _stream(self, x: torch.Tensor) -> torch.Tensor:
         """A private, contiguous copy of the joint sequence in the dtype the residual stream is kept in."""
         dt = torch.float32 if self.cfg.residual_fp32 else torch.bfloat16
@@ -646,6 +662,49 @@ class DMStack(nn.Module):
         for blk, img in zip(self.blocks, cache.images):
             blk(x, temb, self._rot_gen, segs, inplace=True, workspace=self._ws_gen, prefix=(img, P))
         return self._result(x, 0, hidden_states.dim() == 3, return_dict)
+
+
+class GraphedStack:
+    """A recorded ``DMStack.forward``: ``__call__`` copies the inputs into the recorded buffers, replays the graph and
+    returns the recorded outputs ({"sample", "joint"}; overwritten by the next call).  Nothing inside the recording
+    clears memory with a memset node or copies from pageable host memory; the stack's workspaces are the ones the
+    eager path uses, so eager and recorded forwards of one stack must not overlap in time."""
+
+    def __init__(self, stack: "DMStack", inputs: dict, context_cache: Optional["ContextCache"]):
+        if _batch_size(inputs["hidden_states"], 3) != 1:
+            raise NotImplementedError("a graph records one sample; run a batch as a loop over replays")
+        dev = inputs["hidden_states"].device
+        self.stack, self.cache = stack, context_cache
+        self.static = {k: (v.to(dev).clone() if v is not None else None) for k, v in inputs.items()}
+        side = torch.cuda.Stream(device=dev)            # default priority
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(2):                          # allocate workspaces, tables and library handles outside the graph
+                self._run()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.out = self._run()
+
+    def _run(self):
+        return self.stack(return_dict=True, context_cache=self.cache, **self.static)
+
+    def __call__(self, hidden_states: torch.Tensor, timestep: torch.Tensor,
+                 encoder_hidden_states: Optional[torch.Tensor] = None, action_states: Optional[torch.Tensor] = None,
+                 audio_states: Optional[torch.Tensor] = None) -> dict:
+        given = dict(hidden_states=hidden_states, timestep=timestep, encoder_hidden_states=encoder_hidden_states,
+                     action_states=action_states, audio_states=audio_states)
+        for k, v in given.items():
+            dst = self.static[k]
+            if (v is None) != (dst is None):
+                raise ValueError(f"{k}: the graph was recorded {'with' if dst is not None else 'without'} it")
+            if v is not None:
+                if tuple(v.shape) != tuple(dst.shape):
+                    raise ValueError(f"{k}: shape {tuple(v.shape)} differs from the recorded {tuple(dst.shape)}")
+                dst.copy_(v)
+        self.graph.replay()
+        return self.out
 
 
 class DMTransformer(nn.Module):

@@ -684,3 +684,36 @@ def test_transformer_with_audio_stream_and_context_cache():
     n0 = 64 + cfg.n_video
     assert_close(out["audio"][0], y[n0:n0 + 9] @ f(m.audio_proj_out.weight).t() + f(m.audio_proj_out.bias), BF16_COS, BF16_REL, "audio head")
     assert_close(out["action"][0], y[n0 + 9:] @ f(m.action_proj_out.weight).t() + f(m.action_proj_out.bias), BF16_COS, BF16_REL, "action head (after audio)")
+
+
+def test_stack_forward_recorded_as_a_graph():
+    """A forward recorded into a HIP graph (launch-bound shapes): every replay - with the program's own eager work and
+    synchronisations between them, on new inputs - gives the bits of the eager forward; a wrong shape is refused."""
+    cfg = DMConfig("g", 256, 2, 128, 512, 3, (2, 4, 8), n_text=24, n_action=6, n_audio=5, n_branches=4, qk_norm=True)
+    st = DMStack(cfg, device=dev())
+    st.reset_parameters(9)
+    g = torch.Generator(device=dev()).manual_seed(9)
+    with torch.no_grad():
+        for blk in st.blocks:
+            blk.adaLN_modulation.bias.copy_(0.3 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
+    mk = lambda n: torch.randn((1, n, 256), generator=g, device=dev()).to(torch.bfloat16)
+    def inputs():
+        return dict(hidden_states=mk(cfg.n_video), timestep=torch.rand(1, generator=g, device=dev()) * 1000,
+                    encoder_hidden_states=mk(24), action_states=mk(6), audio_states=mk(5))
+    first = inputs()
+    graphed = st.capture(**first)
+    for i in range(4):
+        inp = first if i == 0 else inputs()
+        want = st(return_dict=True, **inp)
+        want = {k: v.clone() for k, v in want.items()}
+        torch.cuda.synchronize()
+        # eager work of other shapes between the replays (its launches must not disturb the recording's buffers)
+        other = DMConfig("o", 256, 2, 128, 512, 1, (1, 4, 8))
+        ops.adaln_rmsnorm(mk(40)[0], torch.ones(256, dtype=torch.bfloat16, device=dev()))
+        got = graphed(**inp)
+        torch.cuda.synchronize()
+        assert torch.equal(got["sample"], want["sample"]) and torch.equal(got["joint"], want["joint"]), f"replay {i}"
+    with pytest.raises(ValueError):
+        graphed(**{**first, "hidden_states": mk(cfg.n_video - 1)})
+    with pytest.raises(ValueError):
+        graphed(**{**first, "audio_states": None})
