@@ -31,6 +31,20 @@ def test_library_exports_every_declared_symbol():
     assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 2 * 128 * 2 * 64 * 2 + 2 * 2 * 4
 
 
+def test_loaded_library_was_built_from_the_present_sources(tmp_path):
+    """The loader never runs a stale build: the library carries the hash of the sources it was built from, readable
+    from the file without loading it, and load() rebuilds the in-tree library when that hash differs."""
+    from cosmos_amd import build as B
+    lib = _lib.load()
+    want = B.source_hash()
+    assert len(want) == 16 and lib.cdm_source_hash().decode() == want
+    assert B.built_hash(_lib.lib_path()) == want
+    stale = tmp_path / "stale.so"
+    stale.write_bytes(b"\x7fELF....CDM_SRC_HASH=0123456789abcdef....")
+    assert B.built_hash(str(stale)) == "0123456789abcdef" != want
+    assert B.built_hash(str(tmp_path / "missing.so")) == ""
+
+
 def test_bad_arguments_are_rejected_on_the_host():
     lib = _lib.load()
     fake = 0x10000   # aligned, never dereferenced: validation fails first

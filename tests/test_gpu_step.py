@@ -155,7 +155,7 @@ def test_denoising_loop_with_transformer_and_stepper():
     lat0 = torch.randn((1, 4, 2, 6, 8), generator=g, device=dev())
 
     def run(batched):
-        st = UniPCStepper(flow_sigmas(4, 3.0), guidance_scale=3.0, solver_order=2)
+        st = UniPCStepper(flow_sigmas(4, 10.0), guidance_scale=3.0, solver_order=2)     # flow_shift of the reference's call site
         lat = lat0.clone()
         for t in st.timesteps:
             ts = torch.tensor([t], device=dev())
@@ -179,3 +179,32 @@ def test_denoising_loop_with_transformer_and_stepper():
     x1 = eu.step(vc.contiguous(), vu.contiguous(), lat0.clone())
     want = lat0 + (eu.sigmas[1] - eu.sigmas[0]) * (vu.float() + 3.0 * (vc.float() - vu.float()))
     assert torch.allclose(x1, want, rtol=1e-5, atol=1e-5)
+
+
+def test_denoising_loop_with_cached_text_context():
+    """The loop of the integration notes under the hybrid mask: the text run's K/V (conditional and null prompt) are
+    packed once and every step carries only the generator tokens; same latents as the loop that re-runs the text."""
+    from cosmos_amd import DMTransformer, UniPCStepper
+    from cosmos_amd.config import DMConfig
+    cfg = DMConfig("loopc", 256, 2, 128, 512, 2, (2, 3, 4), n_text=64, n_branches=2, qk_norm=True, hybrid_mask=True)
+    m = DMTransformer(cfg, latent_channels=4, device=dev())
+    m.reset_parameters(11)
+    g = torch.Generator(device=dev()).manual_seed(11)
+    ctx = torch.randn((1, 64, 256), generator=g, device=dev()).to(torch.bfloat16)
+    null = torch.zeros_like(ctx)
+    lat0 = torch.randn((1, 4, 2, 6, 8), generator=g, device=dev())
+    cache, null_cache = m.stack.precompute_context(ctx), m.stack.precompute_context(null)
+
+    def run(cached):
+        st = UniPCStepper(flow_sigmas(4, 10.0), guidance_scale=3.0, solver_order=2)
+        lat = lat0.clone()
+        for t in st.timesteps:
+            ts = torch.tensor([t], device=dev())
+            vc, = m(lat, ts, encoder_hidden_states=ctx, context_cache=cache if cached else None)
+            vu, = m(lat, ts, encoder_hidden_states=null, context_cache=null_cache if cached else None)
+            st.step(vc.contiguous(), vu.contiguous(), lat)
+        return lat
+
+    a, b = run(True), run(False)
+    assert bool(torch.isfinite(a).all()) and float((a - lat0).abs().max()) > 1e-3
+    assert float((a - b).abs().max()) <= 1e-2 * float(b.abs().max())
