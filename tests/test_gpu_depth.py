@@ -186,4 +186,20 @@ def test_full_size_stack_at_depth(name):
         y = blk(taken[l], temb, rot, segs, workspace=ws)
         want = O.dm_block(taken[l].float().cpu(), oracle_weights(blk, cfg.n_branches), mods_c[l], cos_c, sin_c, cfg.n_heads, segs,
                           attn_rows=rows)
-        assert_close(y[rows.to(dev())], want, *tol, f"{name}: layer {l + 1} of {L} at full size, teacher-forced rows")
+        got = y[rows.to(dev())]
+        if not cfg.fp8:
+            assert_close(got, want, *tol, f"{name}: layer {l + 1} of {L} at full size, teacher-forced rows")
+            continue
+        # e4m3: the adaLN-gated generator rows meet 5e-2 against the UNQUANTISED oracle; the un-gated text rows take the
+        # block's update at full size and are held to the noise of the oracle that quantises at the same places
+        gated = torch.zeros(len(rows), dtype=torch.bool)
+        for (s0, ln, _, modulated) in segs:
+            if modulated:
+                gated |= (rows >= s0) & (rows < s0 + ln)
+        assert_close(got[gated.to(dev())], want[gated], *tol, f"{name}: layer {l + 1} of {L} at full size, teacher-forced gated rows")
+        want8 = O.dm_block(taken[l].float().cpu(), oracle_weights(blk, cfg.n_branches), mods_c[l], cos_c, sin_c, cfg.n_heads, segs,
+                           attn_rows=rows, fp8=True)
+        ung = ~gated
+        noise = O.max_rel_err(want8[ung], want[ung])
+        assert_close(got[ung.to(dev())], want[ung], 0.0, 10.0, f"{name}: layer {l + 1} of {L} at full size, teacher-forced un-gated rows")
+        assert O.max_rel_err(got[ung.to(dev())], want[ung]) < 1.25 * noise and O.max_rel_err(got[ung.to(dev())], want8[ung]) < noise
