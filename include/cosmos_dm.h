@@ -178,7 +178,9 @@ typedef struct cdm_qk_norm {
  *     (cookbooks/cosmos3/cosmos3-model-architecture.png, right panel; README.md:74): the first P tokens (the AR /
  *     text run) attend causally among themselves and to nothing else, every other token attends to all tokens.
  *   workspace: cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim) bytes of caller-owned device memory
- *   (holds K and V re-laid out as 64-key tile images); its contents are undefined afterwards.
+ *   (holds K and V re-laid out as 64-key tile images, followed by one fp32 per K/V head and tile: the largest key
+ *   norm of the tile, from which the kernel bounds the scores of a row and decides whether it needs running row maxima
+ *   at all); its contents are undefined afterwards.
  * head_dim in {64, 128}; n_tokens >= 1 arbitrary.
  */
 int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_kv_heads, int32_t head_dim);
@@ -253,8 +255,11 @@ int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const
                              const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
                              void* stream);
 
-/* Tuning knob for measurements: selects a kernel variant by name ("attn", "gemm"); returns the
- * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default. */
+/* Knob for tests and measurements, process-wide (not per thread or stream): selects a kernel variant by name; returns the
+ * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default of either.
+ *   "attn": 1 = 64 query rows per wave (four waves per workgroup), 2 = the default kernel with per-tile row maxima always
+ *           taken (the default drops them where the norm bound of the scores allows);
+ *   "gemm": 1 = two-stage pipeline instead of the five-slot ring. */
 int32_t cdm_set_variant(const char* op, int32_t variant);
 
 /*
