@@ -44,7 +44,7 @@ __device__ __forceinline__ int key_perm(int i) {
 //    so a score leaves the MFMA already shifted and p = exp2(S) needs no per-score FMA;
 //  * m_ref is a running reference that only moves when a row's tile maximum exceeds it by more than
 //    2^kGrowLog2 (then O and l are rescaled: exact, merely a different reference);
-//  * the row sum uses v_dot2c_f32_bf16 on the packed probabilities (2 values per instruction).
+//  * the row sum adds the fp32 exponentials (v_add_f32); the probabilities are rounded to bf16 once, for the second product.
 // ---------------------------------------------------------------------------------------------
 constexpr float kGrowLog2 = 4.0f;
 
@@ -113,14 +113,17 @@ __device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-// NEED_MAX = false: the caller has shown that no score of this wave's rows can exceed the reference by more than
-//   2^kSafeLog2 (norm bound |q| max|k|), so the per-tile row maximum and the reference update are dropped altogether.
-template <int HD, int QS, bool NEED_MAX, class Mid>
+// BOUND: the kernel has bounded the scores of its rows (|q| max|k|).  Where no score of the wave's rows can exceed the
+//   reference by more than 2^kSafeLog2, need_max (wave-uniform) is false and the per-tile row maximum and the reference
+//   update are skipped altogether; where the bound fails they run in the tail, after block B instead of under its MFMAs
+//   (one loop body for both cases: two copies of the loop do not fit the register budget).
+//   Without BOUND the row maximum is always taken, under the MFMAs of block B.
+template <int HD, int QS, bool BOUND, class Mid>
 __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
                                           f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
                                           f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
-                                          bool next_masked, const int (&next_keys_valid)[QS]) {
+                                          bool next_masked, const int (&next_keys_valid)[QS], bool need_max) {
     constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
     // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot, a second
     // copy of the last tile, and their result is never used - cheaper than a second copy of the step.  When the last
@@ -142,27 +145,26 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
         }
     }
     bf16x8 pf[QS][4];
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
-        float psum = 0.0f;
+        // the row sum adds the fp32 exponentials with plain v_add_f32 (two chains): next to MFMAs a v_dot2c_f32_bf16 on
+        // the packed pairs costs the matrix pipe several times what two adds cost it
+        float psum0 = 0.0f, psum1 = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             bf16x8 p8;
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
-                bf16x2 pp;
                 const float e0 = __builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e]);
                 const float e1 = __builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1]);
-                pp[0] = (__bf16)e0;
-                pp[1] = (__bf16)e1;
-                psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
-                p8[e] = pp[0];
-                p8[e + 1] = pp[1];
+                psum0 += e0;
+                psum1 += e1;
+                p8[e] = (__bf16)e0;
+                p8[e + 1] = (__bf16)e1;
             }
             pf[qs][j] = p8;
         }
-        l_run[qs] += psum;
+        l_run[qs] += psum0 + psum1;
     }
     bf16x8 vw[VWIN];
 #pragma unroll
@@ -200,7 +202,7 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
         if (i + VWIN < NV) vw[i % VWIN] = v_frag<HD>(sv_cur, (i + VWIN) / TS, (i + VWIN) % TS, lane);
     }
     float mx[QS];
-    if constexpr (NEED_MAX) {
+    if constexpr (!BOUND) {
 #pragma unroll
         for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
     }
@@ -209,11 +211,15 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
     for (int i = 0; i < NV * QS; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if constexpr (NEED_MAX) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        if constexpr (!BOUND) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(0);
-    if constexpr (!NEED_MAX) return;
+    if constexpr (BOUND) {
+        if (!need_max) return;
+#pragma unroll
+        for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
+    }
 
     // ---- tail.  mx is relative to the reference (the scores are); moving the reference by d means: O and l
     // shrink by 2^-d, the scores already computed for tile j+1 drop by d, and so does the accumulator seed.
@@ -493,7 +499,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // before barrier j: both tiles are complete at barrier j - 1 (neither is the most recently issued group there),
     // and their slots are not refilled before barrier j + 1.
     const bool late_sync = QS == 1 && wave >= 4;
-#define CDM_ATTN_STEP(SCUR, SNEXT, NEEDMAX)                                                                     \
+#define CDM_ATTN_STEP(SCUR, SNEXT)                                                                              \
     {                                                                                                           \
         const int k_fill = ks_cur;                              /* slot of K(j)   == j % 3     */               \
         const int k_next2 = ks_next == 2 ? 0 : ks_next + 1;     /* slot of K(j+2) == (j+2) % 3 */               \
@@ -508,27 +514,19 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QS];                                                                                         \
         _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS, NEEDMAX>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },         \
+        pipe_step<HD, QS, BOUND>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },               \
                           sk + ks_next * TILE_BYTES, sv + v_cur * TILE_BYTES, sk + k_next2 * TILE_BYTES, qf, kw, \
-                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 >= NT), nvalid);  \
+                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 >= NT), nvalid,   \
+                          need_max);                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         if (late_sync) load_v();                                                                                \
         ks_cur = ks_next;                                                                                       \
         ks_next = ks_next == 2 ? 0 : ks_next + 1;                                                               \
     }
-    // wave-uniform choice; both loops take the same barriers
-    if (need_max) {
-        for (int j = 0; j < NTW; ++j) {
-            CDM_ATTN_STEP(s_a, s_b, true)
-            if (++j >= NTW) break;
-            CDM_ATTN_STEP(s_b, s_a, true)
-        }
-    } else if constexpr (BOUND) {
-        for (int j = 0; j < NTW; ++j) {
-            CDM_ATTN_STEP(s_a, s_b, false)
-            if (++j >= NTW) break;
-            CDM_ATTN_STEP(s_b, s_a, false)
-        }
+    for (int j = 0; j < NTW; ++j) {
+        CDM_ATTN_STEP(s_a, s_b)
+        if (++j >= NTW) break;
+        CDM_ATTN_STEP(s_b, s_a)
     }
 #undef CDM_ATTN_STEP
     // no direct-to-LDS write may outlive the workgroup; after the barrier no wave reads the K / V rings any more and
