@@ -183,9 +183,9 @@ __device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) 
 
 constexpr int kStagePitch = 256 + 16;      // bytes per staged row (16-byte multiple; the pad spreads rows over banks)
 
-// wave-private staging area -> C: COLS (128 or 64) columns of ESIZE bytes (2 = bf16, 4 = fp32) of 128 rows, whole rows
+// wave-private staging area -> C: COLS (128 or 64) columns of ESIZE bytes (2 = bf16, 4 = fp32) of ROWS rows, whole rows
 // per store instruction
-template <int COLS, int ESIZE = 2>
+template <int COLS, int ESIZE = 2, int ROWS = 128>
 __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, const char* stage, int row0, int col0, int lane) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
     constexpr int LPR = COLS * ESIZE / 16;       // lanes per row (16 bytes each)
@@ -193,7 +193,7 @@ __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, con
     const int rl = lane / LPR, ch = lane % LPR;
     const int col = col0 + ch * (16 / ESIZE);
 #pragma unroll
-    for (int it = 0; it < 128 / RPI; ++it) {
+    for (int it = 0; it < ROWS / RPI; ++it) {
         const int rloc = it * RPI + rl;
         const uint4 v = *reinterpret_cast<const uint4*>(stage + rloc * kStagePitch + ch * 16);
         const int row = row0 + rloc;
@@ -208,20 +208,21 @@ __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, con
     }
 }
 
-template <int EPI, bool FP8>
-__device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32x16 (&acc)[4][4], int m0, int n0, int wm,
+// MI = 32-row blocks per wave: 4 (four waves, 128 x 128 each) or 2 (eight waves, 64 x 128 each)
+template <int EPI, bool FP8, int MI = 4>
+__device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32x16 (&acc)[MI][4], int m0, int n0, int wm,
                                          int wn, int lane, char* stage) {
-    // `stage` (optional): kStagePitch * 128 bytes of LDS private to this wave.  The finished bf16 values then go
+    // `stage` (optional): kStagePitch * 32 MI bytes of LDS private to this wave.  The finished bf16 values then go
     // there first and leave as whole rows, 16 bytes per lane: a store instruction covers 4 (SWIGLU: 8) output rows of
     // 256 (128) contiguous bytes instead of 32 rows of 16 bytes.  All workgroups reach their epilogue at about the
     // same time, so the epilogue runs at the HBM write rate; partial-line stores (which left the L2 as several
     // writes per line when the row stride is a large power of two) made it up to four times longer.
     const int r32 = lane & 31, kh = lane >> 5;
-    const int row_base = m0 + wm * 128 + r32;
+    const int row_base = m0 + wm * (32 * MI) + r32;
     if (EPI == CDM_EPI_SWIGLU) {
         const int col_base = n0 + wn * 64 + 4 * kh;      // wave's 128 tile columns = [gate 64 | up 64]
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
+        for (int mi = 0; mi < MI; ++mi) {
             const int row = row_base + mi * 32;
             if (row >= t.m_end) continue;
             const float sr = FP8 ? p.sa[row] : 1.0f;
@@ -248,7 +249,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
                     else *reinterpret_cast<uint2*>(crow + col) = o2;
                 }
         }
-        if (stage) copy_out<64>(p, t, stage, m0 + wm * 128, n0 + wn * 64, lane);
+        if (stage) copy_out<64, 2, 32 * MI>(p, t, stage, m0 + wm * (32 * MI), n0 + wn * 64, lane);
         return;
     }
     const int col_base = n0 + wn * 128 + 4 * kh;
@@ -260,7 +261,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) {
+            for (int mi = 0; mi < MI; ++mi) {
                 const int row = row_base + mi * 32;
                 if (row >= t.m_end) continue;
                 const float sr = FP8 ? p.sa[row] : 1.0f;
@@ -284,14 +285,14 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
                         else *reinterpret_cast<float4*>(C + (int64_t)row * p.ldc + col) = o;
                     }
             }
-            if (stage) copy_out<64, 4>(p, t, stage, m0 + wm * 128, n0 + wn * 128 + 64 * h, lane);
+            if (stage) copy_out<64, 4, 32 * MI>(p, t, stage, m0 + wm * (32 * MI), n0 + wn * 128 + 64 * h, lane);
         }
         return;
     }
     const bool rope = EPI == CDM_EPI_ROPE_QK && n0 + wn * 128 < p.rope_cols;   // wave-uniform: whole heads of Q or K
     const int half = p.head_dim >> 1;
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
         const int row = row_base + mi * 32;
         if (row >= t.m_end) continue;
         if (FP8) {      // rank-1 dequantisation scale on the fp32 accumulators
@@ -353,7 +354,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32
                 else *reinterpret_cast<uint2*>(crow + col) = o2;
             }
     }
-    if (stage) copy_out<128>(p, t, stage, m0 + wm * 128, n0 + wn * 128, lane);
+    if (stage) copy_out<128, 2, 32 * MI>(p, t, stage, m0 + wm * (32 * MI), n0 + wn * 128, lane);
 }
 
 template <int EPI, bool FP8>
@@ -607,6 +608,154 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane, s_ring + wave * (128 * kStagePitch));
 }
 
+// ---------------------------------------------------------------------------------------------
+// The ring pipeline with EIGHT waves (two per SIMD): same 256 x 256 tile, same five-slot ring of 32 KB granules, same
+// swizzle and epilogues; a wave owns 64 x 128 of the tile (2 x 4 accumulator blocks, 128 registers), so two waves fit a
+// SIMD's register file.  A wave that issues a direct-to-LDS load sits in the vector-memory issue queue for a while; with
+// one wave per SIMD the matrix pipe starves meanwhile however carefully the loads are spread, with two the other wave's
+// MFMAs fill the gap.  The price is LDS traffic: 6 fragment reads per 8 MFMAs instead of 8 per 16.
+//   stage t (bf16):  K0 K1 K2 | wait + barrier | K3      Kk = the 8 MFMAs of k-step k, the 6 fragment reads of the next
+//   stage t (e4m3):  K0 | wait + barrier | K1            k-step under the first six of them
+//   loads per wave and k-tile: 4 of A(t+2) ahead of the barrier, 4 of W(t+2) behind it (into the slot of A(t)).
+// ---------------------------------------------------------------------------------------------
+template <bool FP8>
+struct Frags8 {
+    using T = typename std::conditional<FP8, i32x8, bf16x8>::type;
+    T a[2], b[4];
+};
+
+template <int EPI, bool FP8>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_ring8_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(1024))) char s_ring[5 * kGranule];
+
+    Tile tile;
+    if (!locate_tile(p, tile)) return;
+    const int tn = tile.tn;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;          // 4 x 2 waves of 64 x 128
+    const int m0 = tile.m0;
+    const int n0 = (EPI == CDM_EPI_SWIGLU) ? tn * (BN / 2) : tn * BN;
+
+    // per-lane byte offsets of the wave's 4 + 4 loads of one k-tile: load j covers tile rows (8 j + wave) * 8 .. + 7
+    uint32_t oa[4], ob[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = (j * 8 + wave) * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ swz128(row);
+        int am = row;
+        am = (m0 + am) < tile.m_end ? am : tile.m_end - 1 - m0;
+        oa[j] = (uint32_t)(am * (int)p.lda + chunk * 16);
+        // SWIGLU: tile rows come in 64-row groups [gate | up | gate | up]; the rows of load j lie in group j
+        int bn = (EPI == CDM_EPI_SWIGLU) ? (j >> 1) * 64 + (row & 63) : row;
+        bn = (n0 + bn) < p.N ? bn : p.N - 1 - n0;
+        ob[j] = (uint32_t)(bn * (int)p.ldw + chunk * 16);
+    }
+    const char* abase = reinterpret_cast<const char*>(p.A) + (int64_t)m0 * p.lda;
+    const char* wbase = reinterpret_cast<const char*>(tile.W) + (int64_t)n0 * p.ldw;
+    const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(tile.W2) + (int64_t)n0 * p.ldw : wbase;
+    const uint32_t l0 = lds_addr_of(s_ring) + wave * 1024;
+
+    f32x16 acc[2][4];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+    const int KT = p.K / (FP8 ? 128 : 64);   // k-tiles of 128 bytes (at least 2, host-checked)
+    auto gload = [&](int t, int op, int slot, int j) {
+        const int ko = (t < KT ? t : KT - 1) * 128;
+        if (op == 0) {
+            lds_dma16(abase + ko, oa[j], l0 + slot * kGranule + j * 8192);
+        } else {
+            const char* wb = (EPI == CDM_EPI_SWIGLU && (j & 1)) ? w2base : wbase;
+            lds_dma16(wb + ko, ob[j], l0 + slot * kGranule + j * 8192);
+        }
+    };
+    const int r32 = lane & 31, kh = lane >> 5;
+    constexpr int KS = FP8 ? 2 : 4;
+    uint32_t fa[KS], fb[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int chunk = FP8 ? 4 * ks + 2 * kh : 2 * ks + kh;
+        const uint32_t in_row = (uint32_t)(r32 * 128 + ((chunk ^ swz128(r32)) << 4));
+        fa[ks] = in_row + wm * 8192;
+        fb[ks] = in_row + wn * 16384;
+    }
+    auto rd = [&](uint32_t off) {
+        if constexpr (FP8) {
+            const int4 lo = *reinterpret_cast<const int4*>(s_ring + off);
+            const int4 hi = *reinterpret_cast<const int4*>(s_ring + (off ^ 16));
+            return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        } else {
+            return *reinterpret_cast<const bf16x8*>(s_ring + off);
+        }
+    };
+    // fragment q of k-step ks: q = 0 -> a0, 1..4 -> b0..b3, 5 -> a1 (the order the MFMAs need them)
+    auto frag = [&](Frags8<FP8>& f, int slot_a, int slot_b, int ks, int q) {
+        if (q == 0) f.a[0] = rd(fa[ks] + slot_a * kGranule);
+        else if (q <= 4) f.b[q - 1] = rd(fb[ks] + slot_b * kGranule + (q - 1) * 4096);
+        else f.a[1] = rd(fa[ks] + slot_a * kGranule + 4096);
+    };
+    auto mfma = [&](const Frags8<FP8>& f, int i) {
+        const int mi = i >> 2, ni = i & 3;
+        if constexpr (FP8)
+            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[ni], f.a[mi], acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                          0x7f7f7f7f);
+        else
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[ni], f.a[mi], acc[mi][ni], 0, 0, 0);
+    };
+    // prologue: granules 0..3 (tiles 0 and 1)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gload(0, 0, 0, j);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gload(0, 1, 1, j);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gload(1, 0, 2, j);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gload(1, 1, 3, j);
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");     // tile 0 has landed everywhere
+    Frags8<FP8> X, Y;
+#pragma unroll
+    for (int q = 0; q < 6; ++q) frag(X, 0, 1, 0, q);
+
+#define CDM_FENCE __builtin_amdgcn_sched_barrier(0)
+#define CDM_KSTEP8(CUR, NXT, FA, FB, FKS, LOADS)                                                                  \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                               \
+        mfma(CUR, i);                                                                                             \
+        if (i < 6) frag(NXT, FA, FB, FKS, i);                                                                     \
+        LOADS;                                                                                                    \
+        CDM_FENCE;                                                                                                \
+    }
+#define CDM_RING8_BARRIER                                                                                         \
+    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                      \
+    CDM_FENCE;
+    int sa = 0, sb = 1, na = 2, nb = 3, f2 = 4;
+    for (int t = 0; t < KT; ++t) {
+        if constexpr (FP8) {
+            CDM_KSTEP8(X, Y, sa, sb, 1, if (i & 1) gload(t + 2, 0, f2, i >> 1))
+            CDM_RING8_BARRIER
+            CDM_KSTEP8(Y, X, na, nb, 0, if (i & 1) gload(t + 2, 1, sa, i >> 1))
+        } else {
+            CDM_KSTEP8(X, Y, sa, sb, 1, if (i == 3 || i == 7) gload(t + 2, 0, f2, i == 3 ? 0 : 1))
+            CDM_KSTEP8(Y, X, sa, sb, 2, if (i == 3) gload(t + 2, 0, f2, 2))
+            CDM_KSTEP8(X, Y, sa, sb, 3, if (i == 1) gload(t + 2, 0, f2, 3))
+            CDM_RING8_BARRIER
+            CDM_KSTEP8(Y, X, na, nb, 0, if (i & 1) gload(t + 2, 1, sa, i >> 1))
+        }
+        const int o_sa = sa, o_sb = sb;
+        sa = na; sb = nb; na = f2; nb = o_sa; f2 = o_sb;
+    }
+#undef CDM_RING8_BARRIER
+#undef CDM_KSTEP8
+#undef CDM_FENCE
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    epilogue<EPI, FP8, 2>(p, tile, acc, m0, n0, wm, wn, lane, s_ring + wave * (64 * kStagePitch));
+}
+
 // esize = bytes per operand element (2 = bf16, 1 = e4m3); strides in elements
 int32_t validate(const char* who, int esize, const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2,
                  void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epi, const void* R, int64_t ldr,
@@ -658,8 +807,12 @@ template <bool FP8>
 int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epilogue, hipStream_t st, const char* who) {
     const int tile_n = epilogue == CDM_EPI_SWIGLU ? BN / 2 : BN;
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
-    // variant 0 = ring pipeline (default); 1 = two-stage pipeline
-    const bool ring = cdm_get_variant(1) != 1;
+    // variant 0 = ring pipeline, eight waves per workgroup where the reduction is short enough for the epilogue to
+    // matter (K < 16384; measured: the second wave per SIMD hides the epilogue's latencies, the main loop gains
+    // nothing), four otherwise; 1 = two-stage pipeline; 2 / 3 = ring with eight / four waves whatever the shape
+    const int variant = cdm_get_variant(1);
+    const bool ring = variant != 1;
+    const bool ring8 = variant == 2 || (variant == 0 && p.K < 16384);
     int i = 0;
     while (i < n_seg) {
         int ns = 0, total = 0;
@@ -676,7 +829,8 @@ int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epi
         p.n_seg = ns; p.total_tiles = total;
         const int grid = ((total + 7) / 8) * 8;
 #define CDM_LAUNCH(E)                                                         \
-    if (ring) gemm_ring_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p);         \
+    if (ring8) gemm_ring8_kernel<E, FP8><<<grid, 512, 0, st>>>(p);            \
+    else if (ring) gemm_ring_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p);    \
     else gemm_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p)
         switch (epilogue) {
             case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;

@@ -87,7 +87,7 @@ def test_mrope_standalone(hd, H, sections):
 
 
 # ------------------------------------------------------------------ GEMM
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (8, 8, 128), (300, 264, 256), (1024, 3072, 1024), (515, 1000, 384),
                                    (257, 520, 4096), (4100, 4360, 256)])      # the last: 306 tiles, more than the chip has CUs
 def test_gemm_plain(M, N, K, variant):
@@ -115,7 +115,7 @@ def test_gemm_strided_views_and_determinism():
     assert torch.equal(c1, c2)
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 @pytest.mark.parametrize("M,N,K", [(256, 128, 128), (333, 200, 256), (1024, 4096, 1024), (4100, 2184, 256)])
 def test_gemm_swiglu(M, N, K, variant, request):
     prev = ops.set_variant("gemm", variant)
@@ -129,7 +129,7 @@ def test_gemm_swiglu(M, N, K, variant, request):
     assert_close(c, want, 0.99999, 6e-3, f"swiglu {M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 @pytest.mark.parametrize("M,N,K,gated", [(256, 256, 128, True), (300, 1024, 512, True), (77, 264, 128, False),
                                          (4100, 4360, 128, True)])
 def test_gemm_gate_residual(M, N, K, gated, variant, request):
@@ -148,7 +148,7 @@ def test_gemm_gate_residual(M, N, K, gated, variant, request):
     assert torch.equal(r, c)
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 @pytest.mark.parametrize("hd,H,sections", [(64, 4, (16, 24, 24)), (128, 2, (32, 48, 48))])
 def test_gemm_rope_qk(hd, H, sections, variant, request):
     prev = ops.set_variant("gemm", variant)
@@ -183,7 +183,7 @@ def test_grouped_gemm_three_segments():
     assert_close(c, want, 0.99999, 6e-3, "grouped gemm")
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 def test_grouped_gemm_fp8_and_gaps(variant, request):
     """e4m3 grouped launch: three segments with their own weights, one of them empty, rows outside every segment
     untouched; the long segment spans several row tiles so the short ones share its grid."""
@@ -217,7 +217,7 @@ def test_grouped_gemm_fp8_and_gaps(variant, request):
     assert torch.equal(out, ref)
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 @pytest.mark.parametrize("M,N,K,gated,fp8", [(256, 256, 128, True, False), (300, 1024, 512, True, False), (77, 264, 128, False, False),
                                              (515, 520, 256, True, True), (1030, 4096, 1024, True, False)])
 def test_gemm_gate_residual_fp32_stream(M, N, K, gated, fp8, variant, request):
@@ -496,7 +496,7 @@ def test_adaln_rmsnorm_quant():
     assert torch.equal(s, s2) and torch.equal(yq.float(), q2.float())
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3])
 @pytest.mark.parametrize("M,N,K,epi", [(256, 256, 256, "none"), (300, 520, 512, "none"), (300, 264, 256, "swiglu"),
                                        (130, 256, 256, "gate_residual"), (515, 1000, 1792, "none"),
                                        (4100, 4360, 256, "none"), (4100, 2184, 256, "swiglu")])
