@@ -208,153 +208,173 @@ __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, con
     }
 }
 
-// MI = 32-row blocks per wave: 4 (four waves, 128 x 128 each) or 2 (eight waves, 64 x 128 each)
-template <int EPI, bool FP8, int MI = 4>
-__device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, f32x16 (&acc)[MI][4], int m0, int n0, int wm,
-                                         int wn, int lane, char* stage) {
-    // `stage` (optional): kStagePitch * 32 MI bytes of LDS private to this wave.  The finished bf16 values then go
+// Views of a wave's accumulators: where in the wave's ROWS x 128 piece of the tile a lane's quads (four consecutive
+// columns of one row) sit.  RS row slots x CS column slots per lane; column slot cs + CS / 2 is 64 columns right of cs.
+template <int MI>
+struct Acc32 {      // MI x 4 blocks of 32 x 32 (v_mfma_*_32x32x*): lane = row % 32 + 32 kh, quads at columns 8 g + 4 kh
+    f32x16 (&v)[MI][4];
+    static constexpr int RS = MI, CS = 16, ROWS = 32 * MI;
+    static __device__ __forceinline__ int row_local(int rs, int lane) { return rs * 32 + (lane & 31); }
+    static __device__ __forceinline__ int col_local(int cs, int lane) { return (cs >> 2) * 32 + (cs & 3) * 8 + (lane >> 5) * 4; }
+    __device__ __forceinline__ float get(int rs, int cs, int e) const { return v[rs][cs >> 2][4 * (cs & 3) + e]; }
+    __device__ __forceinline__ void set(int rs, int cs, int e, float x) { v[rs][cs >> 2][4 * (cs & 3) + e] = x; }
+};
+template <int MI>
+struct Acc16 {      // MI x 8 blocks of 16 x 16 (v_mfma_*_16x16x*): lane = row % 16 + 16 q, one quad per block at column 4 q
+    f32x4 (&v)[MI][8];
+    static constexpr int RS = MI, CS = 8, ROWS = 16 * MI;
+    static __device__ __forceinline__ int row_local(int rs, int lane) { return rs * 16 + (lane & 15); }
+    static __device__ __forceinline__ int col_local(int cs, int lane) { return cs * 16 + (lane >> 4) * 4; }
+    __device__ __forceinline__ float get(int rs, int cs, int e) const { return v[rs][cs][e]; }
+    __device__ __forceinline__ void set(int rs, int cs, int e, float x) { v[rs][cs][e] = x; }
+};
+
+// row0 = first row of the wave's piece of the tile; the piece covers tile columns wn * 128 .. + 127
+template <int EPI, bool FP8, class ACC>
+__device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC acc, int row0, int n0, int wn, int lane,
+                                         char* stage) {
+    // `stage` (optional): kStagePitch * ROWS bytes of LDS private to this wave.  The finished bf16 values then go
     // there first and leave as whole rows, 16 bytes per lane: a store instruction covers 4 (SWIGLU: 8) output rows of
     // 256 (128) contiguous bytes instead of 32 rows of 16 bytes.  All workgroups reach their epilogue at about the
     // same time, so the epilogue runs at the HBM write rate; partial-line stores (which left the L2 as several
     // writes per line when the row stride is a large power of two) made it up to four times longer.
-    const int r32 = lane & 31, kh = lane >> 5;
-    const int row_base = m0 + wm * (32 * MI) + r32;
+    constexpr int RS = ACC::RS, CS = ACC::CS, ROWS = ACC::ROWS, HALF = CS / 2, QUARTER = CS / 4;
     if (EPI == CDM_EPI_SWIGLU) {
-        const int col_base = n0 + wn * 64 + 4 * kh;      // wave's 128 tile columns = [gate 64 | up 64]
+        const int colw = n0 + wn * 64;       // wave's 128 tile columns = [gate 64 | up 64] of output columns colw .. + 63
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) {
-            const int row = row_base + mi * 32;
+        for (int rs = 0; rs < RS; ++rs) {
+            const int rl = ACC::row_local(rs, lane), row = row0 + rl;
             if (row >= t.m_end) continue;
             const float sr = FP8 ? p.sa[row] : 1.0f;
             bf16_t* crow = p.C + (int64_t)row * p.ldc;
 #pragma unroll
-            for (int nj = 0; nj < 2; ++nj)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int col = col_base + nj * 32 + 8 * g;
-                    if (col >= p.N) continue;
-                    float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
-                    if (FP8) {
-                        const float4 a = *reinterpret_cast<const float4*>(t.sw + col);
-                        const float4 b = *reinterpret_cast<const float4*>(t.sw2 + col);
-                        sg[0] = a.x * sr; sg[1] = a.y * sr; sg[2] = a.z * sr; sg[3] = a.w * sr;
-                        su[0] = b.x * sr; su[1] = b.y * sr; su[2] = b.z * sr; su[3] = b.w * sr;
-                    }
-                    float o[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        o[e] = silu_f(acc[mi][nj][4 * g + e] * sg[e]) * (acc[mi][nj + 2][4 * g + e] * su[e]);
-                    const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
-                    if (stage) *reinterpret_cast<uint2*>(stage + (mi * 32 + r32) * kStagePitch + (nj * 32 + 8 * g + 4 * kh) * 2) = o2;
-                    else *reinterpret_cast<uint2*>(crow + col) = o2;
+            for (int cs = 0; cs < HALF; ++cs) {
+                const int cl = ACC::col_local(cs, lane), col = colw + cl;
+                if (col >= p.N) continue;
+                float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
+                if (FP8) {
+                    const float4 a = *reinterpret_cast<const float4*>(t.sw + col);
+                    const float4 b = *reinterpret_cast<const float4*>(t.sw2 + col);
+                    sg[0] = a.x * sr; sg[1] = a.y * sr; sg[2] = a.z * sr; sg[3] = a.w * sr;
+                    su[0] = b.x * sr; su[1] = b.y * sr; su[2] = b.z * sr; su[3] = b.w * sr;
                 }
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = silu_f(acc.get(rs, cs, e) * sg[e]) * (acc.get(rs, cs + HALF, e) * su[e]);
+                const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
+                if (stage) *reinterpret_cast<uint2*>(stage + rl * kStagePitch + cl * 2) = o2;
+                else *reinterpret_cast<uint2*>(crow + col) = o2;
+            }
         }
-        if (stage) copy_out<64, 2, 32 * MI>(p, t, stage, m0 + wm * (32 * MI), n0 + wn * 64, lane);
+        if (stage) copy_out<64, 2, ROWS>(p, t, stage, row0, colw, lane);
         return;
     }
-    const int col_base = n0 + wn * 128 + 4 * kh;
+    const int colw = n0 + wn * 128;
     if (EPI == CDM_EPI_GATE_RESIDUAL_F32) {
-        // the residual stream in fp32: R and C are float rows (in place when they coincide).  A wave's 128 x 128
-        // result goes through its staging area 64 columns (256 bytes per row) at a time.
+        // the residual stream in fp32: R and C are float rows (in place when they coincide).  The wave's result goes
+        // through its staging area 64 columns (256 bytes per row) at a time.
         float* C = reinterpret_cast<float*>(p.C);
         const float* R = reinterpret_cast<const float*>(p.R);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi) {
-                const int row = row_base + mi * 32;
+            for (int rs = 0; rs < RS; ++rs) {
+                const int rl = ACC::row_local(rs, lane), row = row0 + rl;
                 if (row >= t.m_end) continue;
                 const float sr = FP8 ? p.sa[row] : 1.0f;
 #pragma unroll
-                for (int nj = 0; nj < 2; ++nj)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int ni = 2 * h + nj;
-                        const int col = col_base + ni * 32 + 8 * g;
-                        if (col >= p.N) continue;
-                        const float4 r4 = *reinterpret_cast<const float4*>(R + (int64_t)row * p.ldr + col);
-                        float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
-                        if (t.gate) g4 = *reinterpret_cast<const float4*>(t.gate + col);
-                        if (FP8) {
-                            const float4 w4 = *reinterpret_cast<const float4*>(t.sw + col);
-                            g4.x *= sr * w4.x; g4.y *= sr * w4.y; g4.z *= sr * w4.z; g4.w *= sr * w4.w;
-                        }
-                        const float4 o = make_float4(r4.x + g4.x * acc[mi][ni][4 * g], r4.y + g4.y * acc[mi][ni][4 * g + 1],
-                                                     r4.z + g4.z * acc[mi][ni][4 * g + 2], r4.w + g4.w * acc[mi][ni][4 * g + 3]);
-                        if (stage) *reinterpret_cast<float4*>(stage + (mi * 32 + r32) * kStagePitch + (nj * 32 + 8 * g + 4 * kh) * 4) = o;
-                        else *reinterpret_cast<float4*>(C + (int64_t)row * p.ldc + col) = o;
+                for (int c = 0; c < HALF; ++c) {
+                    const int cs = h * HALF + c;
+                    const int cl = ACC::col_local(cs, lane), col = colw + cl;
+                    if (col >= p.N) continue;
+                    const float4 r4 = *reinterpret_cast<const float4*>(R + (int64_t)row * p.ldr + col);
+                    float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
+                    if (t.gate) g4 = *reinterpret_cast<const float4*>(t.gate + col);
+                    if (FP8) {
+                        const float4 w4 = *reinterpret_cast<const float4*>(t.sw + col);
+                        g4.x *= sr * w4.x; g4.y *= sr * w4.y; g4.z *= sr * w4.z; g4.w *= sr * w4.w;
                     }
+                    const float4 o = make_float4(r4.x + g4.x * acc.get(rs, cs, 0), r4.y + g4.y * acc.get(rs, cs, 1),
+                                                 r4.z + g4.z * acc.get(rs, cs, 2), r4.w + g4.w * acc.get(rs, cs, 3));
+                    if (stage) *reinterpret_cast<float4*>(stage + rl * kStagePitch + (cl - 64 * h) * 4) = o;
+                    else *reinterpret_cast<float4*>(C + (int64_t)row * p.ldc + col) = o;
+                }
             }
-            if (stage) copy_out<64, 4, 32 * MI>(p, t, stage, m0 + wm * (32 * MI), n0 + wn * 128 + 64 * h, lane);
+            if (stage) copy_out<64, 4, ROWS>(p, t, stage, row0, colw + 64 * h, lane);
         }
         return;
     }
-    const bool rope = EPI == CDM_EPI_ROPE_QK && n0 + wn * 128 < p.rope_cols;   // wave-uniform: whole heads of Q or K
+    const bool rope = EPI == CDM_EPI_ROPE_QK && colw < p.rope_cols;   // wave-uniform: whole heads of Q or K
     const int half = p.head_dim >> 1;
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
-        const int row = row_base + mi * 32;
+    for (int rs = 0; rs < RS; ++rs) {
+        const int rl = ACC::row_local(rs, lane), row = row0 + rl;
         if (row >= t.m_end) continue;
         if (FP8) {      // rank-1 dequantisation scale on the fp32 accumulators
             const float sr = p.sa[row];
 #pragma unroll
-            for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int col = col_base + ni * 32 + 8 * g;
-                    const float4 w4 = col < p.N ? *reinterpret_cast<const float4*>(t.sw + col) : make_float4(0, 0, 0, 0);
-                    acc[mi][ni][4 * g + 0] *= sr * w4.x;
-                    acc[mi][ni][4 * g + 1] *= sr * w4.y;
-                    acc[mi][ni][4 * g + 2] *= sr * w4.z;
-                    acc[mi][ni][4 * g + 3] *= sr * w4.w;
-                }
+            for (int cs = 0; cs < CS; ++cs) {
+                const int col = colw + ACC::col_local(cs, lane);
+                const float4 w4 = col < p.N ? *reinterpret_cast<const float4*>(t.sw + col) : make_float4(0, 0, 0, 0);
+                acc.set(rs, cs, 0, acc.get(rs, cs, 0) * (sr * w4.x));
+                acc.set(rs, cs, 1, acc.get(rs, cs, 1) * (sr * w4.y));
+                acc.set(rs, cs, 2, acc.get(rs, cs, 2) * (sr * w4.z));
+                acc.set(rs, cs, 3, acc.get(rs, cs, 3) * (sr * w4.w));
+            }
         }
         if (EPI == CDM_EPI_ROPE_QK && rope) {
-            // rotate-half pairs (i, i + head_dim/2).  head_dim 128: blocks (nj, nj + 2), pair index 32 nj + ...;
-            // head_dim 64: two heads per wave, blocks (nj, nj + 1) with nj even, pair index inside the block
+            // rotate-half pairs (i, i + head_dim/2).  head_dim 128: the wave's columns are one head, column slots
+            // (c, c + CS/2), pair index = the column of c; head_dim 64: two heads per wave, slots (lo, lo + CS/4)
+            // with lo in the first half of either head, pair index = the column inside the head
             const float* cr = p.cos + (int64_t)row * half;
             const float* sr_ = p.sin + (int64_t)row * half;
 #pragma unroll
-            for (int nj = 0; nj < 2; ++nj)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int lo = p.head_dim == 128 ? nj : 2 * nj, hi = p.head_dim == 128 ? nj + 2 : 2 * nj + 1;
-                    const int i = (p.head_dim == 128 ? nj * 32 : 0) + 8 * g + 4 * kh;
-                    const float4 c4 = *reinterpret_cast<const float4*>(cr + i);
-                    const float4 s4 = *reinterpret_cast<const float4*>(sr_ + i);
-                    const float c[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
+            for (int c = 0; c < HALF; ++c) {
+                const bool hd128 = p.head_dim == 128;
+                const int lo128 = c, lo64 = (c / QUARTER) * HALF + (c % QUARTER);
+                const int i = hd128 ? ACC::col_local(lo128, lane) : (ACC::col_local(lo64, lane) & 31);
+                const float4 c4 = *reinterpret_cast<const float4*>(cr + i);
+                const float4 s4 = *reinterpret_cast<const float4*>(sr_ + i);
+                const float cc[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
+                if (hd128) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float x1 = acc[mi][lo][4 * g + e], x2 = acc[mi][hi][4 * g + e];
-                        acc[mi][lo][4 * g + e] = x1 * c[e] - x2 * sn[e];
-                        acc[mi][hi][4 * g + e] = x2 * c[e] + x1 * sn[e];
+                        const float x1 = acc.get(rs, lo128, e), x2 = acc.get(rs, lo128 + HALF, e);
+                        acc.set(rs, lo128, e, x1 * cc[e] - x2 * sn[e]);
+                        acc.set(rs, lo128 + HALF, e, x2 * cc[e] + x1 * sn[e]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float x1 = acc.get(rs, lo64, e), x2 = acc.get(rs, lo64 + QUARTER, e);
+                        acc.set(rs, lo64, e, x1 * cc[e] - x2 * sn[e]);
+                        acc.set(rs, lo64 + QUARTER, e, x2 * cc[e] + x1 * sn[e]);
                     }
                 }
+            }
         }
         bf16_t* crow = p.C + (int64_t)row * p.ldc;
         const bf16_t* rrow = EPI == CDM_EPI_GATE_RESIDUAL ? p.R + (int64_t)row * p.ldr : nullptr;
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int col = col_base + ni * 32 + 8 * g;
-                if (col >= p.N) continue;
-                float o[4] = {acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]};
-                if (EPI == CDM_EPI_GATE_RESIDUAL) {
-                    const uint2 r2 = *reinterpret_cast<const uint2*>(rrow + col);
-                    float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
-                    if (t.gate) g4 = *reinterpret_cast<const float4*>(t.gate + col);
-                    o[0] = bf16lo(r2.x) + g4.x * o[0];
-                    o[1] = bf16hi(r2.x) + g4.y * o[1];
-                    o[2] = bf16lo(r2.y) + g4.z * o[2];
-                    o[3] = bf16hi(r2.y) + g4.w * o[3];
-                }
-                const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
-                if (stage) *reinterpret_cast<uint2*>(stage + (mi * 32 + r32) * kStagePitch + (ni * 32 + 8 * g + 4 * kh) * 2) = o2;
-                else *reinterpret_cast<uint2*>(crow + col) = o2;
+        for (int cs = 0; cs < CS; ++cs) {
+            const int cl = ACC::col_local(cs, lane), col = colw + cl;
+            if (col >= p.N) continue;
+            float o[4] = {acc.get(rs, cs, 0), acc.get(rs, cs, 1), acc.get(rs, cs, 2), acc.get(rs, cs, 3)};
+            if (EPI == CDM_EPI_GATE_RESIDUAL) {
+                const uint2 r2 = *reinterpret_cast<const uint2*>(rrow + col);
+                float4 g4 = make_float4(1.f, 1.f, 1.f, 1.f);
+                if (t.gate) g4 = *reinterpret_cast<const float4*>(t.gate + col);
+                o[0] = bf16lo(r2.x) + g4.x * o[0];
+                o[1] = bf16hi(r2.x) + g4.y * o[1];
+                o[2] = bf16lo(r2.y) + g4.z * o[2];
+                o[3] = bf16hi(r2.y) + g4.w * o[3];
             }
+            const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
+            if (stage) *reinterpret_cast<uint2*>(stage + rl * kStagePitch + cl * 2) = o2;
+            else *reinterpret_cast<uint2*>(crow + col) = o2;
+        }
     }
-    if (stage) copy_out<128, 2, 32 * MI>(p, t, stage, m0 + wm * (32 * MI), n0 + wn * 128, lane);
+    if (stage) copy_out<128, 2, ROWS>(p, t, stage, row0, colw, lane);
 }
 
 template <int EPI, bool FP8>
@@ -427,7 +447,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         compute_stage<FP8>(sa1, sb1, acc, wm, wn, lane);
     }
 
-    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane, nullptr);
+    epilogue<EPI, FP8>(p, tile, Acc32<4>{acc}, m0 + wm * 128, n0, wn, lane, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -605,24 +625,27 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     // surplus loads must not outlive the workgroup's LDS; after the barrier no wave reads the ring any more and
     // each wave owns a quarter of it as the staging area of its epilogue
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    epilogue<EPI, FP8>(p, tile, acc, m0, n0, wm, wn, lane, s_ring + wave * (128 * kStagePitch));
+    epilogue<EPI, FP8>(p, tile, Acc32<4>{acc}, m0 + wm * 128, n0, wn, lane, s_ring + wave * (128 * kStagePitch));
 }
 
 // ---------------------------------------------------------------------------------------------
-// The ring pipeline with EIGHT waves (two per SIMD): same 256 x 256 tile, same five-slot ring of 32 KB granules, same
-// swizzle and epilogues; a wave owns 64 x 128 of the tile (2 x 4 accumulator blocks, 128 registers), so two waves fit a
-// SIMD's register file.  A wave that issues a direct-to-LDS load sits in the vector-memory issue queue for a while; with
-// one wave per SIMD the matrix pipe starves meanwhile however carefully the loads are spread, with two the other wave's
-// MFMAs fill the gap.  The price is LDS traffic: 6 fragment reads per 8 MFMAs instead of 8 per 16.
-//   stage t (bf16):  K0 K1 K2 | wait + barrier | K3      Kk = the 8 MFMAs of k-step k, the 6 fragment reads of the next
-//   stage t (e4m3):  K0 | wait + barrier | K1            k-step under the first six of them
-//   loads per wave and k-tile: 4 of A(t+2) ahead of the barrier, 4 of W(t+2) behind it (into the slot of A(t)).
+// The ring pipeline with EIGHT waves (two per SIMD) and 16 x 16 MFMAs: same 256 x 256 tile, same five-slot ring of 32 KB
+// granules, same epilogues; a wave owns 64 x 128 of the tile as 4 x 8 accumulator blocks of 16 x 16 (128 registers).
+//  * v_mfma_f32_16x16x32_bf16 moves a fifth fewer register bytes per flop than 32x32x16 (half the accumulator traffic,
+//    twice the operand traffic) and the chip runs into its power limit, not its issue rate, on random operands: a loop of
+//    nothing but MFMAs sustains 9 % more with the small shape, and this kernel 6 - 11 % more than its 32 x 32 twin.
+//  * The second wave of a SIMD feeds the matrix pipe while the first sits in the vector-memory issue queue with a
+//    direct-to-LDS load, or in the latencies of its epilogue.
+//  * k-step = 32 MFMAs, order: W block ni outer, A block mi inner.  The four A fragments of the NEXT k-step are read under
+//    MFMAs 18 - 30 (two register sets), the W fragments stream through a four-entry window two blocks ahead, so a k-step
+//    reads 12 fragments for 32 MFMAs.  bf16: two k-steps per k-tile (K 32 each); e4m3: one (K 128).
+//  * The window makes the reads of k-tile t reach into its last k-step (until MFMA 20), so the wait + barrier ("every wave
+//    has finished reading tile t, and tile t+1 has landed") sits at MFMA 22 of it; the fragments of tile t+1 that the
+//    next k-step starts with are read right behind it.  A(t+2) goes out ahead of the barrier, into the slot that W(t-1)
+//    left at the previous barrier; W(t+2) behind it, into the slot of A(t).
+// The swizzle of a ring row differs from the four-wave kernel's: a fragment read covers 16 rows x 4 chunks here.
 // ---------------------------------------------------------------------------------------------
-template <bool FP8>
-struct Frags8 {
-    using T = typename std::conditional<FP8, i32x8, bf16x8>::type;
-    T a[2], b[4];
-};
+__device__ __forceinline__ int swz16(int row) { return (row >> 1) & 7; }
 
 template <int EPI, bool FP8>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_ring8_kernel(const GemmParams p) {
@@ -643,7 +666,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int row = (j * 8 + wave) * 8 + (lane >> 3);
-        const int chunk = (lane & 7) ^ swz128(row);
+        const int chunk = (lane & 7) ^ swz16(row);
         int am = row;
         am = (m0 + am) < tile.m_end ? am : tile.m_end - 1 - m0;
         oa[j] = (uint32_t)(am * (int)p.lda + chunk * 16);
@@ -657,13 +680,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const char* w2base = EPI == CDM_EPI_SWIGLU ? reinterpret_cast<const char*>(tile.W2) + (int64_t)n0 * p.ldw : wbase;
     const uint32_t l0 = lds_addr_of(s_ring) + wave * 1024;
 
-    f32x16 acc[2][4];
+    f32x4 acc[4][8];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+        for (int ni = 0; ni < 8; ++ni) acc[mi][ni] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int KT = p.K / (FP8 ? 128 : 64);   // k-tiles of 128 bytes (at least 2, host-checked)
     auto gload = [&](int t, int op, int slot, int j) {
@@ -675,13 +696,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             lds_dma16(wb + ko, ob[j], l0 + slot * kGranule + j * 8192);
         }
     };
-    const int r32 = lane & 31, kh = lane >> 5;
-    constexpr int KS = FP8 ? 2 : 4;
+    using T = typename std::conditional<FP8, i32x8, bf16x8>::type;
+    constexpr int KS = FP8 ? 1 : 2;
+    const int r16 = lane & 15, q = lane >> 4;
     uint32_t fa[KS], fb[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        const int chunk = FP8 ? 4 * ks + 2 * kh : 2 * ks + kh;
-        const uint32_t in_row = (uint32_t)(r32 * 128 + ((chunk ^ swz128(r32)) << 4));
+        // bf16: 16-byte chunk 4 ks + q of the row; e4m3: chunks 2 q and 2 q + 1 (the second at the address ^ 16)
+        const int chunk = FP8 ? 2 * q : 4 * ks + q;
+        const uint32_t in_row = (uint32_t)(r16 * 128 + ((chunk ^ swz16(r16)) << 4));
         fa[ks] = in_row + wm * 8192;
         fb[ks] = in_row + wn * 16384;
     }
@@ -694,20 +717,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             return *reinterpret_cast<const bf16x8*>(s_ring + off);
         }
     };
-    // fragment q of k-step ks: q = 0 -> a0, 1..4 -> b0..b3, 5 -> a1 (the order the MFMAs need them)
-    auto frag = [&](Frags8<FP8>& f, int slot_a, int slot_b, int ks, int q) {
-        if (q == 0) f.a[0] = rd(fa[ks] + slot_a * kGranule);
-        else if (q <= 4) f.b[q - 1] = rd(fb[ks] + slot_b * kGranule + (q - 1) * 4096);
-        else f.a[1] = rd(fa[ks] + slot_a * kGranule + 4096);
-    };
-    auto mfma = [&](const Frags8<FP8>& f, int i) {
-        const int mi = i >> 2, ni = i & 3;
-        if constexpr (FP8)
-            acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[ni], f.a[mi], acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                          0x7f7f7f7f);
-        else
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[ni], f.a[mi], acc[mi][ni], 0, 0, 0);
-    };
+    auto afrag = [&](int slot, int ks, int mi) { return rd(fa[ks] + slot * kGranule + mi * 2048); };
+    auto bfrag = [&](int slot, int ks, int ni) { return rd(fb[ks] + slot * kGranule + ni * 2048); };
+
     // prologue: granules 0..3 (tiles 0 and 1)
 #pragma unroll
     for (int j = 0; j < 4; ++j) gload(0, 0, 0, j);
@@ -718,42 +730,86 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int j = 0; j < 4; ++j) gload(1, 1, 3, j);
     asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");     // tile 0 has landed everywhere
-    Frags8<FP8> X, Y;
+    T X[4], Y[4], B[4];
 #pragma unroll
-    for (int q = 0; q < 6; ++q) frag(X, 0, 1, 0, q);
+    for (int mi = 0; mi < 4; ++mi) X[mi] = afrag(0, 0, mi);
+    B[0] = bfrag(1, 0, 0);
+    B[1] = bfrag(1, 0, 1);
 
-#define CDM_FENCE __builtin_amdgcn_sched_barrier(0)
-#define CDM_KSTEP8(CUR, NXT, FA, FB, FKS, LOADS)                                                                  \
-    _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                               \
-        mfma(CUR, i);                                                                                             \
-        if (i < 6) frag(NXT, FA, FB, FKS, i);                                                                     \
-        LOADS;                                                                                                    \
-        CDM_FENCE;                                                                                                \
-    }
-#define CDM_RING8_BARRIER                                                                                         \
-    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                      \
-    CDM_FENCE;
     int sa = 0, sb = 1, na = 2, nb = 3, f2 = 4;
-    for (int t = 0; t < KT; ++t) {
-        if constexpr (FP8) {
-            CDM_KSTEP8(X, Y, sa, sb, 1, if (i & 1) gload(t + 2, 0, f2, i >> 1))
-            CDM_RING8_BARRIER
-            CDM_KSTEP8(Y, X, na, nb, 0, if (i & 1) gload(t + 2, 1, sa, i >> 1))
-        } else {
-            CDM_KSTEP8(X, Y, sa, sb, 1, if (i == 3 || i == 7) gload(t + 2, 0, f2, i == 3 ? 0 : 1))
-            CDM_KSTEP8(Y, X, sa, sb, 2, if (i == 3) gload(t + 2, 0, f2, 2))
-            CDM_KSTEP8(X, Y, sa, sb, 3, if (i == 1) gload(t + 2, 0, f2, 3))
-            CDM_RING8_BARRIER
-            CDM_KSTEP8(Y, X, na, nb, 0, if (i & 1) gload(t + 2, 1, sa, i >> 1))
+    int t = 0;
+    // LAST = the k-step that ends k-tile t (the only one of an e4m3 tile, the second of a bf16 tile)
+    auto kstep = [&](auto last_c, T (&cur)[4], T (&nxt)[4]) {
+        constexpr bool LAST = decltype(last_c)::value;
+        constexpr int ks = LAST ? KS - 1 : 0;           // k-step of the W fragments in flight
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int ni = i >> 2, mi = i & 3;
+            if constexpr (FP8)
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(B[ni & 3], cur[mi], acc[mi][ni], 0 /*A: e4m3*/,
+                                                                               0 /*B: e4m3*/, 0, 0x7f7f7f7f /*scale 1*/, 0,
+                                                                               0x7f7f7f7f);
+            else
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B[ni & 3], cur[mi], acc[mi][ni], 0, 0, 0);
+            if (!LAST) {
+                if (mi == 0) B[(ni + 2) & 3] = ni < 6 ? bfrag(sb, 0, ni + 2) : bfrag(sb, 1, ni - 6);
+                if (i >= 18 && (i & 3) == 2) nxt[(i - 18) >> 2] = afrag(sa, 1, (i - 18) >> 2);
+                if (i == 9) gload(t + 2, 0, f2, 0);
+                if (i == 25) gload(t + 2, 0, f2, 1);
+            } else {
+                if (mi == 0 && ni < 6) B[(ni + 2) & 3] = bfrag(sb, ks, ni + 2);
+                if constexpr (FP8) {
+                    if (i == 3) gload(t + 2, 0, f2, 0);
+                    if (i == 9) gload(t + 2, 0, f2, 1);
+                    if (i == 15) gload(t + 2, 0, f2, 2);
+                    if (i == 19) gload(t + 2, 0, f2, 3);
+                } else {
+                    if (i == 5) gload(t + 2, 0, f2, 2);
+                    if (i == 13) gload(t + 2, 0, f2, 3);
+                }
+                if (i == 22) {
+                    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                    nxt[0] = afrag(na, 0, 0);
+                }
+                if (i == 23) nxt[1] = afrag(na, 0, 1);
+                if (i == 24) B[0] = bfrag(nb, 0, 0);
+                if (i == 25) nxt[2] = afrag(na, 0, 2);
+                if (i == 26) nxt[3] = afrag(na, 0, 3);
+                if (i == 27) gload(t + 2, 1, sa, 0);
+                if (i == 28) B[1] = bfrag(nb, 0, 1);
+                if (i == 29) gload(t + 2, 1, sa, 1);
+                if (i == 30) gload(t + 2, 1, sa, 2);
+                if (i == 31) gload(t + 2, 1, sa, 3);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    auto rotate = [&]() {
         const int o_sa = sa, o_sb = sb;
         sa = na; sb = nb; na = f2; nb = o_sa; f2 = o_sb;
+        ++t;
+    };
+    if constexpr (FP8) {
+        while (t < KT) {
+            kstep(std::true_type{}, X, Y);
+            rotate();
+            if (t < KT) {
+                kstep(std::true_type{}, Y, X);
+                rotate();
+            }
+        }
+    } else {
+        while (t < KT) {
+            kstep(std::false_type{}, X, Y);
+            kstep(std::true_type{}, Y, X);
+            rotate();
+        }
     }
-#undef CDM_RING8_BARRIER
-#undef CDM_KSTEP8
-#undef CDM_FENCE
+    // surplus loads must not outlive the workgroup's LDS; after the barrier no wave reads the ring any more and
+    // each wave owns an eighth of it as the staging area of its epilogue
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    epilogue<EPI, FP8, 2>(p, tile, acc, m0, n0, wm, wn, lane, s_ring + wave * (64 * kStagePitch));
+    epilogue<EPI, FP8>(p, tile, Acc16<4>{acc}, m0 + wm * 64, n0, wn, lane, s_ring + wave * (64 * kStagePitch));
 }
 
 // esize = bytes per operand element (2 = bf16, 1 = e4m3); strides in elements
@@ -807,12 +863,11 @@ template <bool FP8>
 int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epilogue, hipStream_t st, const char* who) {
     const int tile_n = epilogue == CDM_EPI_SWIGLU ? BN / 2 : BN;
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
-    // variant 0 = ring pipeline, eight waves per workgroup where the reduction is short enough for the epilogue to
-    // matter (K < 16384; measured: the second wave per SIMD hides the epilogue's latencies, the main loop gains
-    // nothing), four otherwise; 1 = two-stage pipeline; 2 / 3 = ring with eight / four waves whatever the shape
+    // variant 0 = ring pipeline with eight waves and 16 x 16 MFMAs; 1 = two-stage pipeline, four waves, 32 x 32 MFMAs;
+    // 3 = ring pipeline with four waves and 32 x 32 MFMAs (2 = 0)
     const int variant = cdm_get_variant(1);
     const bool ring = variant != 1;
-    const bool ring8 = variant == 2 || (variant == 0 && p.K < 16384);
+    const bool ring8 = variant == 0 || variant == 2;
     int i = 0;
     while (i < n_seg) {
         int ns = 0, total = 0;

@@ -259,8 +259,8 @@ int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const
  * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default of either.
  *   "attn": 1 = 64 query rows per wave (four waves per workgroup), 2 = the default kernel with per-tile row maxima always
  *           taken (the default drops them where the norm bound of the scores allows);
- *   "gemm": 1 = two-stage pipeline instead of the five-slot ring; 2 / 3 = the ring with eight / four waves per workgroup
- *           whatever the shape (the default takes eight where K < 16384). */
+ *   "gemm": 1 = two-stage pipeline with four waves and 32 x 32 MFMAs, 3 = five-slot ring with four waves and 32 x 32 MFMAs,
+ *           instead of the five-slot ring with eight waves and 16 x 16 MFMAs. */
 int32_t cdm_set_variant(const char* op, int32_t variant);
 
 /*
