@@ -3,14 +3,14 @@
 // earlier call, per-head RMSNorm of Q and K.
 //
 // Work split: one workgroup owns 256 query rows of one head and streams all keys in tiles of 64.
-// Scores are computed TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_32x32x16_bf16: the A operand is a K
-// tile row (plain 16-byte LDS read), the B operand is Q held in registers for the whole kernel.  In
-// the accumulator layout every lane then owns ONE query column and 16 keys per 32-key block, so the
-// row max / row sum of the online softmax are in-lane reductions plus one exchange between the two
-// half-waves.  The probabilities never move between lanes: packed to bf16 they are already the B
-// operand of O^T += V^T . P^T, whose A operand is a row of V^T.  The K rows of a 32-key block are
-// fetched in a permuted order so that the 8 keys a lane holds in accumulator registers 8j..8j+7 are
-// the 8 consecutive keys the second product expects.
+// Scores are computed TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_16x16x32_bf16 (the small shape moves a fifth fewer
+// register bytes per flop than 32x32x16, and on random operands the chip is bound by its power limit): the A operand
+// is a K tile row (plain 16-byte LDS read), the B operand is Q held in registers for the whole kernel.  In the
+// accumulator layout every lane then owns ONE query column and 4 keys per 16-key block, so the row max / row sum of
+// the online softmax are in-lane reductions plus two exchanges between the four quarter-waves.  The probabilities
+// never move between lanes: packed to bf16, the lane's values of key blocks 2s and 2s + 1 are its 8 k-values of the B
+// operand of O^T += V^T . P^T for the 32-key step s, whose A operand is a row of V^T; the V^T image lists the keys of
+// a step in that order (lane quarter g, element e: keys 32 s + 4 g + e and 32 s + 16 + 4 g + e, e = 0..3).
 // Rotate-half mRoPE (and the QK-RMSNorm ahead of it) is applied in registers: to K while it is re-tiled for the
 // kernel, to Q when the kernel loads its Q fragments (both members of a rotary pair sit in the same lane).
 #include <mutex>
@@ -21,24 +21,21 @@ namespace {
 
 constexpr int BN = 64;       // keys per tile
 constexpr int BMQ = 256;     // query rows per workgroup
+constexpr int KB = BN / 16;  // 16-key blocks per tile
 typedef __attribute__((address_space(3))) void lds_void;
-
-// row permutation inside a 32-key block: MFMA output row i holds key pi(i)
-__device__ __forceinline__ int key_perm(int i) {
-    const int g = i >> 3, b = (i >> 2) & 1, r = i & 3;
-    return 16 * (g >> 1) + 8 * b + 4 * (g & 1) + r;
-}
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 // ---------------------------------------------------------------------------------------------
 // Software-pipelined kernel over PRE-TILED K and V.
 //  * K and V are first re-laid out in the workspace as the exact LDS image of each 64-key tile,
 //    chunk-major:  Kp[head][tile][c = dh/8][key r = 0..63][8 ch]   and
-//                  Vp[head][tile][c = key/8 (0..7)][channel row = 0..HD-1][8 keys]  (V transposed).
+//                  Vp[head][tile][c = 0..7][channel row = 0..HD-1][8 keys]  (V transposed; chunk c = 4 s + g holds
+//                  keys 32 s + 4 g + {0..3} and 32 s + 16 + 4 g + {0..3}).
 //    A tile is then one contiguous 16 KB (HD=128) stream for the direct-to-LDS loads, every fragment
 //    read is  lane_base + compile-time offset  (no swizzle arithmetic, two address registers in
 //    total) and 16 consecutive lanes always read 16 distinct 16-byte slots (no bank conflicts).
 //    Keys beyond n_tokens are zero in the workspace and masked to -inf in the last tile.
-//  * the scores of tile j+1 (S^T = K Q^T, 16 MFMAs) are issued BEFORE the softmax of tile j, so one
+//  * the scores of tile j+1 (S^T = K Q^T, 32 MFMAs) are issued BEFORE the softmax of tile j, so one
 //    wave always has matrix work in flight under its own exp/convert VALU work;
 //  * Q is pre-multiplied by log2(e)/sqrt(dh) and the score accumulators start at -m_ref instead of 0,
 //    so a score leaves the MFMA already shifted and p = exp2(S) needs no per-score FMA;
@@ -48,196 +45,191 @@ __device__ __forceinline__ int key_perm(int i) {
 // ---------------------------------------------------------------------------------------------
 constexpr float kGrowLog2 = 4.0f;
 
-// K fragment of k-step ks, key block kvb: lane reads key row pi(lane%32) (+32 for the second block), chunk 2ks + lane/32
+// K fragment of k-step ks (32 channels), key block kb: lane reads key row 16 kb + lane % 16, chunk 4 ks + lane / 16
 template <int HD>
-__device__ __forceinline__ bf16x8 k_frag(const char* sk, int ks, int kvb, int lane) {
-    return *reinterpret_cast<const bf16x8*>(sk + (lane >> 5) * 1024 + key_perm(lane & 31) * 16 + ks * 2048 + kvb * 512);
+__device__ __forceinline__ bf16x8 k_frag(const char* sk, int ks, int kb, int lane) {
+    return *reinterpret_cast<const bf16x8*>(sk + (lane >> 4) * 1024 + (lane & 15) * 16 + ks * 4096 + kb * 256);
 }
-// V^T fragment of key chunk pair j (keys 16j..16j+15), channel block t: lane reads channel row 32t + lane%32, chunk 2j + lane/32
+// V^T fragment of key step s (32 keys), channel block hb: lane reads channel row 16 hb + lane % 16, chunk 4 s + lane / 16
 template <int HD>
-__device__ __forceinline__ bf16x8 v_frag(const char* sv, int j, int t, int lane) {
-    return *reinterpret_cast<const bf16x8*>(sv + (lane >> 5) * (HD * 16) + (lane & 31) * 16 + j * (HD * 32) + t * 512);
+__device__ __forceinline__ bf16x8 v_frag(const char* sv, int s, int hb, int lane) {
+    return *reinterpret_cast<const bf16x8*>(sv + (lane >> 4) * (HD * 16) + (lane & 15) * 16 + s * (HD * 64) + hb * 256);
 }
 
 // Whole score tile with plain just-in-time fragment reads (prologue only).
-template <int HD>
-__device__ __forceinline__ void scores_tile(const char* sk, const bf16x8 (&qf)[HD / 16], f32x16 (&s)[2], int lane) {
+template <int HD, int QB>
+__device__ __forceinline__ void scores_tile(const char* sk, const bf16x8 (&qf)[QB][HD / 32], f32x4 (&s)[KB][QB], int lane) {
 #pragma unroll
-    for (int ks = 0; ks < HD / 16; ++ks)
+    for (int ks = 0; ks < HD / 32; ++ks)
 #pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-            s[kvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag<HD>(sk, ks, kvb, lane), qf[ks], s[kvb], 0, 0, 0);
-}
-
-constexpr int KWIN = 4;     // k-steps of K fragments kept in flight (x2 key blocks)
-constexpr int VWIN = 8;     // V^T fragments kept in flight
-
-template <int HD>
-__device__ __forceinline__ void preload_k(const char* sk, bf16x8 (&kw)[KWIN][2], int lane) {
+        for (int kb = 0; kb < KB; ++kb) {
+            const bf16x8 kf = k_frag<HD>(sk, ks, kb, lane);
 #pragma unroll
-    for (int ks = 0; ks < KWIN; ++ks) {
-        kw[ks][0] = k_frag<HD>(sk, ks, 0, lane);
-        kw[ks][1] = k_frag<HD>(sk, ks, 1, lane);
-    }
-}
-
-// Scores of keys >= keys_valid (ragged last tile) become -inf.  Register v of block kvb holds key
-// 32 kvb + 16 (v/8) + 8 (lane/32) + v%8: the compile-time part is compared against ONE per-lane threshold so that
-// no per-register key index is ever materialised.
-__device__ __forceinline__ void mask_scores(f32x16 (&s)[2], int keys_valid, int lane) {
-    const int thr = keys_valid - 8 * (lane >> 5);
-#pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int kc = 32 * kvb + 16 * (v >> 3) + (v & 7);
-            s[kvb][v] = (kc >= thr) ? -INFINITY : s[kvb][v];
+            for (int qb = 0; qb < QB; ++qb) s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qb][ks], s[kb][qb], 0, 0, 0);
         }
 }
 
-__device__ __forceinline__ float tile_row_max(const f32x16 (&s)[2]) {
-    float mx = __builtin_fmaxf(s[0][0], s[1][0]);
+constexpr int KWIN = 2;     // k-steps of K fragments kept in flight (x4 key blocks)
+constexpr int VWIN = 8;     // V^T fragments kept in flight
+
+template <int HD>
+__device__ __forceinline__ void preload_k(const char* sk, bf16x8 (&kw)[KWIN][KB], int lane) {
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = __builtin_fmaxf(__builtin_fmaxf(mx, s[0][v]), s[1][v]);   // v_max3_f32
+    for (int ks = 0; ks < KWIN; ++ks)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) kw[ks][kb] = k_frag<HD>(sk, ks, kb, lane);
+}
+
+// Scores of keys >= keys_valid[qb] (ragged last tile, causal rows) become -inf.  Register e of key block kb holds key
+// 16 kb + 4 (lane / 16) + e: the compile-time part is compared against ONE per-lane threshold so that no per-register
+// key index is ever materialised.
+template <int QB>
+__device__ __forceinline__ void mask_scores(f32x4 (&s)[KB][QB], const int (&keys_valid)[QB], int lane) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int thr = keys_valid[qb] - 4 * (lane >> 4);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[kb][qb][e] = (16 * kb + e >= thr) ? -INFINITY : s[kb][qb][e];
+    }
+}
+
+template <int QB>
+__device__ __forceinline__ float tile_row_max(const f32x4 (&s)[KB][QB], int qb) {
+    float mx = __builtin_fmaxf(s[0][qb][0], s[0][qb][1]);
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int e = (kb == 0 ? 2 : 0); e < 4; e += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, s[kb][qb][e]), s[kb][qb][e + 1]);   // v_max3_f32
+    mx = __builtin_fmaxf(mx, __shfl_xor(mx, 16, 64));
     return __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
 }
 
 // One pipeline step.  Everything the first MFMAs need is already in registers when the workgroup barrier at
 // the top of the step releases the wave, and all softmax arithmetic is placed under MFMAs:
-//   block A  : S(j+1) = K(j+1) Q^T - m_ref, 16 MFMAs seeded with -m_ref (rolling K fragment window, first
+//   block A  : S(j+1) = K(j+1) Q^T - m_ref, 32 MFMAs seeded with -m_ref (rolling K fragment window, first
 //              KWIN k-steps preloaded in the previous step)
 //              ||  p = exp2(s_cur), bf16 pack, row sum of tile j ; first V^T fragments of tile j (a wave that
 //              takes the step's barrier behind block A reads them before that barrier: V(j) is complete one
 //              barrier early)
-//   block B  : O^T += V^T P^T, 16 MFMAs (rolling V^T window)
+//   block B  : O^T += V^T P^T, 32 MFMAs (rolling V^T window)
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-// BOUND: the kernel has bounded the scores of its rows (|q| max|k|).  Where no score of the wave's rows can exceed the
+// The kernel has bounded the scores of its rows (|q| max|k|).  Where no score of the wave's rows can exceed the
 //   reference by more than 2^kSafeLog2, need_max (wave-uniform) is false and the per-tile row maximum and the reference
-//   update are skipped altogether; where the bound fails they run in the tail, after block B instead of under its MFMAs
-//   (one loop body for both cases: two copies of the loop do not fit the register budget).
-//   Without BOUND the row maximum is always taken, under the MFMAs of block B.
-template <int HD, int QS, bool BOUND, class Mid>
+//   update are skipped altogether; where the bound fails they run in the tail, after block B (one loop body for both
+//   cases: two copies of the loop do not fit the register budget).
+template <int HD, int QB, class Mid>
 __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
-                                          const bf16x8 (&qf)[QS][HD / 16], bf16x8 (&kw)[KWIN][2],
-                                          f32x16 (&s_cur)[QS][2], f32x16 (&s_next)[QS][2],
-                                          f32x16 (&oacc)[QS][HD / 32], f32x16 (&negm)[QS], float (&l_run)[QS], int lane,
-                                          bool next_masked, const int (&next_keys_valid)[QS], bool need_max) {
-    constexpr int KS = HD / 16, TS = HD / 32, NV = 4 * TS;
+                                          const bf16x8 (&qf)[QB][HD / 32], bf16x8 (&kw)[KWIN][KB],
+                                          f32x4 (&s_cur)[KB][QB], f32x4 (&s_next)[KB][QB],
+                                          f32x4 (&oacc)[HD / 16][QB], f32x4 (&negm)[QB], float (&l_run)[QB], int lane,
+                                          bool next_masked, const int (&next_keys_valid)[QB], bool need_max) {
+    constexpr int KS = HD / 32, HB = HD / 16, NV = 2 * HB;
+    // Both blocks are written as a sequence of slots, one MFMA each, fenced so that the compiler keeps them: an odd
+    // slot carries one fragment read, an even slot (head_dim 64: every slot) one piece of the softmax arithmetic.
     // ---- block A.  (In the very last step there is no next tile: the MFMAs then chew on a stale K slot, a second
     // copy of the last tile, and their result is never used - cheaper than a second copy of the step.  When the last
     // tile is ragged that step masks all of its scores like the one before it masked the padding: the zero keys of the
     // padding would otherwise show up as scores of -m_ref, and with every real logit far below zero the tail would
     // move the reference up to them and scale O and l towards zero.)
+    constexpr int NA = KS * KB * QB;              // MFMAs of block A
+    constexpr int NREFILL = (KS - KWIN) * KB;     // K fragments read inside block A
+    constexpr int NSM = QB * 8;                   // softmax pieces: 2 exp, 2 add, 1 pack each
+    constexpr int SMI = NA / NSM;                 // one softmax piece every SMI slots (2 at head_dim 128, 1 at 64)
+    static_assert(SMI >= 1 && NREFILL + (VWIN < NV ? VWIN : NV) <= NA / 2 + NREFILL, "block A has too few slots");
+    u32x4 pw[QB][2];       // the probabilities, packed: B operands of block B
+    bf16x8 vw[VWIN];
+    float psum0[QB], psum1[QB];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
+    for (int qb = 0; qb < QB; ++qb) psum0[qb] = psum1[qb] = 0.0f;
+    int n_v = 0;       // V^T fragments read so far (compile-time after unrolling)
 #pragma unroll
-        for (int qs = 0; qs < QS; ++qs) {
-            s_next[qs][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][0], qf[qs][ks],
-                                                                    ks == 0 ? negm[qs] : s_next[qs][0], 0, 0, 0);
-            s_next[qs][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kw[ks % KWIN][1], qf[qs][ks],
-                                                                    ks == 0 ? negm[qs] : s_next[qs][1], 0, 0, 0);
-        }
-        if (ks + KWIN < KS) {
-            kw[ks % KWIN][0] = k_frag<HD>(sk_next, ks + KWIN, 0, lane);
-            kw[ks % KWIN][1] = k_frag<HD>(sk_next, ks + KWIN, 1, lane);
-        }
-    }
-    bf16x8 pf[QS][4];
-#pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
+    for (int i = 0; i < NA; ++i) {
+        const int ks = i / (KB * QB), kb = (i / QB) % KB, qb = i % QB;
+        s_next[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kw[ks % KWIN][kb], qf[qb][ks],
+                                                                 ks == 0 ? negm[qb] : s_next[kb][qb], 0, 0, 0);
         // the row sum adds the fp32 exponentials with plain v_add_f32 (two chains): next to MFMAs a v_dot2c_f32_bf16 on
         // the packed pairs costs the matrix pipe several times what two adds cost it
-        float psum0 = 0.0f, psum1 = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            bf16x8 p8;
-#pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                const float e0 = __builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e]);
-                const float e1 = __builtin_amdgcn_exp2f(s_cur[qs][j >> 1][8 * (j & 1) + e + 1]);
-                psum0 += e0;
-                psum1 += e1;
-                p8[e] = (__bf16)e0;
-                p8[e + 1] = (__bf16)e1;
-            }
-            pf[qs][j] = p8;
+        if (i % SMI == 0 && i / SMI < NSM) {
+            const int m = i / SMI, q = m / 8, st = (m / 4) % 2, h = (m / 2) % 2, e = 2 * (m % 2);
+            // the empty asm statements tie the piece to its slot: left alone the compiler gathers all exponentials and
+            // conversions of the tile in one place (behind the MFMAs of this block), where nothing overlaps them
+            if (e == 0) asm volatile("" : "+v"(s_cur[2 * st + h][q]));
+            const float e0 = __builtin_amdgcn_exp2f(s_cur[2 * st + h][q][e]);
+            const float e1 = __builtin_amdgcn_exp2f(s_cur[2 * st + h][q][e + 1]);
+            psum0[q] += e0;
+            psum1[q] += e1;
+            uint32_t w = pack_bf16x2(e0, e1);
+            asm volatile("" : "+v"(w), "+v"(psum0[q]), "+v"(psum1[q]));
+            pw[q][st][2 * h + e / 2] = w;
         }
-        l_run[qs] += psum0 + psum1;
+        // a K fragment is replaced right behind its last MFMA; the first V^T fragments follow
+        if (qb == QB - 1 && ks + KWIN < KS) {
+            kw[ks % KWIN][kb] = k_frag<HD>(sk_next, ks + KWIN, kb, lane);
+        } else if (i % 2 == 1 && n_v < VWIN && n_v < NV) {
+            vw[n_v] = v_frag<HD>(sv_cur, n_v / HB, n_v % HB, lane);
+            ++n_v;
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
-    bf16x8 vw[VWIN];
 #pragma unroll
-    for (int i = 0; i < VWIN && i < NV; ++i) vw[i] = v_frag<HD>(sv_cur, i / TS, i % TS, lane);
-    // per MFMA (at most) one fragment read and six VALU instructions
+    for (; n_v < VWIN && n_v < NV; ++n_v) vw[n_v] = v_frag<HD>(sv_cur, n_v / HB, n_v % HB, lane);
 #pragma unroll
-    for (int i = 0; i < 2 * KS * QS; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-    }
-    // the probabilities must be complete here: without this the compiler sinks the whole exp/pack sequence past
-    // the branch below into block B, where it no longer fits under the MFMAs
-#pragma unroll
-    for (int qs = 0; qs < QS; ++qs)
-        asm volatile("" : "+v"(pf[qs][0]), "+v"(pf[qs][1]), "+v"(pf[qs][2]), "+v"(pf[qs][3]), "+v"(l_run[qs]));
+    for (int qb = 0; qb < QB; ++qb) l_run[qb] += psum0[qb] + psum1[qb];
     __builtin_amdgcn_sched_barrier(0);
     mid();                 // the step's synchronisation point for the waves that take it between the two blocks
     __builtin_amdgcn_sched_barrier(0);
-    if (next_masked) {     // wave-uniform: before a ragged last tile, and in every step of a causal query block
-#pragma unroll
-        for (int qs = 0; qs < QS; ++qs) mask_scores(s_next[qs], next_keys_valid[qs], lane);
-    }
+    if (next_masked)       // wave-uniform: before a ragged last tile, and in every step of a causal query block
+        mask_scores<QB>(s_next, next_keys_valid, lane);
 
     // ---- block B.  It is pure matrix work, while the other wave of the SIMD is in its VALU-heavy block A at this
     // time: with the wave's priority raised for the duration, its MFMAs win the issue slot and the other wave's
     // VALU work fills the gaps (0.6 % faster than equal priorities)
     __builtin_amdgcn_s_setprio(1);
+    constexpr int NB = NV * QB;                   // MFMAs of block B
+    static_assert((NV > VWIN ? NV - VWIN : 0) + KWIN * KB <= NB, "block B has too few slots");
+    int n_kpre = 0;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int j = i / TS, t = i % TS;
-#pragma unroll
-        for (int qs = 0; qs < QS; ++qs)
-            oacc[qs][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vw[i % VWIN], pf[qs][j], oacc[qs][t], 0, 0, 0);
-        if (i + VWIN < NV) vw[i % VWIN] = v_frag<HD>(sv_cur, (i + VWIN) / TS, (i + VWIN) % TS, lane);
+    for (int i = 0; i < NB; ++i) {
+        const int f = i / QB, st = f / HB, hb = f % HB, qb = i % QB;
+        oacc[hb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vw[f % VWIN], __builtin_bit_cast(bf16x8, pw[qb][st]), oacc[hb][qb], 0, 0, 0);
+        if (qb == QB - 1 && f + VWIN < NV) {
+            vw[f % VWIN] = v_frag<HD>(sv_cur, (f + VWIN) / HB, (f + VWIN) % HB, lane);
+        } else if (i % 2 == 1 && n_kpre < KWIN * KB && (f + VWIN >= NV || qb != QB - 1)) {
+            kw[n_kpre / KB][n_kpre % KB] = k_frag<HD>(sk_next2, n_kpre / KB, n_kpre % KB, lane);
+            ++n_kpre;
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
-    float mx[QS];
-    if constexpr (!BOUND) {
 #pragma unroll
-        for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
-    }
-    preload_k<HD>(sk_next2, kw, lane);
-#pragma unroll
-    for (int i = 0; i < NV * QS; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if constexpr (!BOUND) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-    }
+    for (; n_kpre < KWIN * KB; ++n_kpre) kw[n_kpre / KB][n_kpre % KB] = k_frag<HD>(sk_next2, n_kpre / KB, n_kpre % KB, lane);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(0);
-    if constexpr (BOUND) {
-        if (!need_max) return;
+    if (!need_max) return;
+    float mx[QB];
 #pragma unroll
-        for (int qs = 0; qs < QS; ++qs) mx[qs] = tile_row_max(s_next[qs]);
-    }
+    for (int qb = 0; qb < QB; ++qb) mx[qb] = tile_row_max<QB>(s_next, qb);
 
     // ---- tail.  mx is relative to the reference (the scores are); moving the reference by d means: O and l
     // shrink by 2^-d, the scores already computed for tile j+1 drop by d, and so does the accumulator seed.
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
-        if (__builtin_amdgcn_ballot_w64(mx[qs] > kGrowLog2) != 0) {
-            const float d = mx[qs] > kGrowLog2 ? mx[qs] : 0.0f;
+    for (int qb = 0; qb < QB; ++qb) {
+        if (__builtin_amdgcn_ballot_w64(mx[qb] > kGrowLog2) != 0) {
+            const float d = mx[qb] > kGrowLog2 ? mx[qb] : 0.0f;
             const float fac = __builtin_amdgcn_exp2f(-d);
-            l_run[qs] *= fac;
+            l_run[qb] *= fac;
 #pragma unroll
-            for (int t = 0; t < TS; ++t)
+            for (int hb = 0; hb < HB; ++hb)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) oacc[qs][t][v] *= fac;
+                for (int e = 0; e < 4; ++e) oacc[hb][qb][e] *= fac;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                s_next[qs][0][v] -= d;
-                s_next[qs][1][v] -= d;
-                negm[qs][v] -= d;
+            for (int e = 0; e < 4; ++e) {
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s_next[kb][qb][e] -= d;
+                negm[qb][e] -= d;
             }
         }
     }
@@ -273,19 +265,21 @@ struct PackedParams {
     QkNormDev qn;                          // optional per-head RMSNorm of Q, applied before the rotation
     int n_tokens, n_heads, n_qblocks;
     int kv_group;                // query heads per K / V head (1 = multi-head attention)
+    int always_max;              // cross-check: take the row maxima of every tile whatever the norm bound says
     float scale_log2e;
 };
 
-// QS = query sub-tiles (of 32 rows) per wave: QS = 1 -> 8 waves, two per SIMD, 256 registers each;
+// QS = query sub-tiles (of 32 rows = two 16-row blocks) per wave: QS = 1 -> 8 waves, two per SIMD, 256 registers each;
 // QS = 2 -> 4 waves, one per SIMD with the 512-register budget; every K / V^T fragment read from LDS then feeds
-// two MFMAs instead of one.
+// four MFMAs instead of two.
 constexpr float kSafeLog2 = 60.0f;      // largest excess over the reference that needs no reference update
 
-// BOUND: take the norm bound of the scores (below) and run the loop without row maxima where it allows
-template <int HD, int QS, bool BOUND>
+template <int HD, int QS>
 __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS, 2 / QS))) void attn_fwd_pipe_kernel(
     const PackedParams p) {
     constexpr int NW = 8 / QS;
+    constexpr int QB = 2 * QS;                         // 16-row query blocks per wave
+    constexpr int KS = HD / 32, HB = HD / 16;
     constexpr int TILE_BYTES = BN * HD * 2;            // same for K and V tiles
     constexpr int PER_WAVE = TILE_BYTES / 1024 / NW;   // direct-to-LDS instructions per wave per tile
     // K(t) lives in slot t % 3 and V(t) in slot t % 4.  V is loaded one step further ahead than its first use by
@@ -297,7 +291,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r32 = lane & 31, kh = lane >> 5;
+    const int r16 = lane & 15, g4 = lane >> 4;
     // XCD-aware placement: workgroup ids are dealt round-robin over the 8 XCDs.  All query blocks of a head go to
     // ONE XCD, so a head's K / V tile images are fetched into one L2 instead of eight, and an XCD owns a contiguous
     // range of heads, so the query heads that share a K / V head (grouped-query attention) share an L2 as well.
@@ -315,12 +309,12 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     const int q0 = qblk * BMQ + wave * (32 * QS);
 
     // ---- Q fragments: rotate-half mRoPE (if tables are given) and the factor log2(e)/sqrt(HD), both in fp32 and
-    // with ONE rounding to bf16.  The lane holds channels 16ks + 8kh .. +7 of its query row for every ks, so
-    // the partner of a channel in k-step ks (< KS/2) is the same register element of k-step ks + KS/2.
+    // with ONE rounding to bf16.  The lane holds channels 32ks + 8g .. +7 (g = lane / 16) of its query row for every
+    // ks, so the partner of a channel in k-step ks (< KS/2) is the same register element of k-step ks + KS/2.
     // An upper bound of every score of a row: |q| max_k |k| (Cauchy-Schwarz on the very bf16 values the
     // matrix cores multiply).  kmax_all = the largest key norm of this K/V head over all tiles, prefix included.
     float kmax_all = 0.0f;
-    if constexpr (BOUND) {
+    {
         const int nm = (p.n_tokens + BN - 1) / BN;
         const float* km = p.kmax + (int64_t)kv_head * nm;
         for (int i = lane; i < nm; i += 64) kmax_all = fmaxf(kmax_all, km[i]);
@@ -328,18 +322,17 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         for (int i = lane; i < p.n_prefix_tiles; i += 64) kmax_all = fmaxf(kmax_all, kmp[i]);
         kmax_all = wave_max(kmax_all);
     }
-    float qnorm[QS];
-    bf16x8 qf[QS][HD / 16];
+    float qnorm[QB];
+    bf16x8 qf[QB][KS];
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
-        constexpr int KS = HD / 16;
-        int qrow = q0 + qs * 32 + r32;
+    for (int qb = 0; qb < QB; ++qb) {
+        int qrow = q0 + qb * 16 + r16;
         qrow = qrow < p.n_tokens ? qrow : p.n_tokens - 1;
-        const bf16_t* qp = p.q + (int64_t)qrow * p.ldq + head * HD + 8 * kh;
+        const bf16_t* qp = p.q + (int64_t)qrow * p.ldq + head * HD + 8 * g4;
         uint4 raw[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qp + 16 * ks);
-        // per-head RMSNorm: the lane holds 8 channels per k-step, its partner (lane ^ 32) the other 8
+        for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+        // per-head RMSNorm: the lane holds 8 channels per k-step, the other three quarter-waves the rest of the row
         float rnorm = 1.0f;
         const float* nw = nullptr;
         if (p.qn.w != nullptr) {
@@ -350,9 +343,10 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
 #pragma unroll
                 for (int j = 0; j < 4; ++j) { const float a = bf16lo(w[j]), b = bf16hi(w[j]); ss += a * a + b * b; }
             }
+            ss += __shfl_xor(ss, 16, 64);
             ss += __shfl_xor(ss, 32, 64);
             rnorm = rsqrtf(ss * (1.0f / HD) + p.qn.eps);
-            nw = p.qn.row(qrow, HD) + 8 * kh;
+            nw = p.qn.row(qrow, HD) + 8 * g4;
         }
 #pragma unroll
         for (int ks = 0; ks < KS / 2; ++ks) {
@@ -361,13 +355,13 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             float n1[8], n2[8];      // norm factors of the channels of k-step ks and of its rotary partners
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                n1[e] = nw ? rnorm * nw[16 * ks + e] : 1.0f;
-                n2[e] = nw ? rnorm * nw[16 * (ks + KS / 2) + e] : 1.0f;
+                n1[e] = nw ? rnorm * nw[32 * ks + e] : 1.0f;
+                n2[e] = nw ? rnorm * nw[32 * (ks + KS / 2) + e] : 1.0f;
             }
             float c[8], sn[8];
             if (p.cos != nullptr) {
-                const float4* cp = reinterpret_cast<const float4*>(p.cos + (int64_t)qrow * (HD / 2) + 16 * ks + 8 * kh);
-                const float4* sp = reinterpret_cast<const float4*>(p.sin + (int64_t)qrow * (HD / 2) + 16 * ks + 8 * kh);
+                const float4* cp = reinterpret_cast<const float4*>(p.cos + (int64_t)qrow * (HD / 2) + 32 * ks + 8 * g4);
+                const float4* sp = reinterpret_cast<const float4*>(p.sin + (int64_t)qrow * (HD / 2) + 32 * ks + 8 * g4);
                 const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
                 c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
                 sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
@@ -385,38 +379,36 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
                 o2[j] = pack_bf16x2((b0 * c[2 * j] + a0 * sn[2 * j]) * p.scale_log2e,
                                     (b1 * c[2 * j + 1] + a1 * sn[2 * j + 1]) * p.scale_log2e);
             }
-            qf[qs][ks] = __builtin_bit_cast(bf16x8, make_uint4(o1[0], o1[1], o1[2], o1[3]));
-            qf[qs][ks + KS / 2] = __builtin_bit_cast(bf16x8, make_uint4(o2[0], o2[1], o2[2], o2[3]));
+            qf[qb][ks] = __builtin_bit_cast(bf16x8, make_uint4(o1[0], o1[1], o1[2], o1[3]));
+            qf[qb][ks + KS / 2] = __builtin_bit_cast(bf16x8, make_uint4(o2[0], o2[1], o2[2], o2[3]));
         }
-        qnorm[qs] = 0.0f;
-        if constexpr (BOUND) {      // norm of the scaled, rotated, rounded query row (the lane and lane ^ 32 hold half each)
+        {      // norm of the scaled, rotated, rounded query row (a quarter of it in each quarter-wave)
             float ss = 0.0f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const uint4 u = __builtin_bit_cast(uint4, qf[qs][ks]);
+                const uint4 u = __builtin_bit_cast(uint4, qf[qb][ks]);
                 const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) { const float a = bf16lo(w[j]), b = bf16hi(w[j]); ss += a * a + b * b; }
             }
+            ss += __shfl_xor(ss, 16, 64);
             ss += __shfl_xor(ss, 32, 64);
-            qnorm[qs] = sqrtf(ss);
+            qnorm[qb] = sqrtf(ss);
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // Q is in registers: from here on vmcnt counts tile loads only
 
-    f32x16 oacc[QS][HD / 32];
-    // negm = minus the softmax reference of the lane's query row (log2 units), replicated over a 16-register
+    f32x4 oacc[HB][QB];
+    // negm = minus the softmax reference of the lane's query row (log2 units), replicated over a 4-register
     // block so that it can seed the score accumulators: the MFMAs then deliver s - m_ref and no subtraction is
     // left in the exp path
-    f32x16 negm[QS];
-    float l_run[QS];
+    f32x4 negm[QB];
+    float l_run[QB];
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
-        l_run[qs] = 0.0f;
+    for (int qb = 0; qb < QB; ++qb) {
+        l_run[qb] = 0.0f;
 #pragma unroll
-        for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[qs][t][v] = 0.0f;
+        for (int hb = 0; hb < HB; ++hb) oacc[hb][qb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
     // key tiles: NP whole tiles of the prefix images, then the NM tiles of the main images
@@ -428,11 +420,11 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // own last row, and every tile it visits is masked per row
     const int b0 = qblk * BMQ;
     const bool causal_wg = b0 < p.causal_prefix;
-    int klim[QS];
+    int klim[QB];
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
-        const int qrow = q0 + qs * 32 + r32;
-        klim[qs] = qrow < p.causal_prefix ? qrow + 1 : n_keys;
+    for (int qb = 0; qb < QB; ++qb) {
+        const int qrow = q0 + qb * 16 + r16;
+        klim[qb] = qrow < p.causal_prefix ? qrow + 1 : n_keys;
     }
     const int kmax = (causal_wg && b0 + BMQ <= p.causal_prefix) ? (b0 + BMQ < n_keys ? b0 + BMQ : n_keys) : n_keys;
     const int NTW = (kmax + BN - 1) / BN;
@@ -461,28 +453,29 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     issue(vbase, vpre, sv_addr, 1, 1);
     issue(vbase, vpre, sv_addr, 2, 2);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(3 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
-    f32x16 s_a[QS][2], s_b[QS][2];      // score tiles ping-pong between the two halves of the unrolled loop
+    f32x4 s_a[KB][QB], s_b[KB][QB];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
-    bool need_max = !BOUND;
+    bool need_max = p.always_max != 0;
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { s_a[qs][0][v] = 0.0f; s_a[qs][1][v] = 0.0f; }
-        scores_tile<HD>(sk, qf[qs], s_a[qs], lane);
-        if (causal_wg || (NT == 1 && ragged)) mask_scores(s_a[qs], klim[qs], lane);
-        const float m0 = tile_row_max(s_a[qs]);      // exact first reference: every row has at least one finite score
+        for (int qb = 0; qb < QB; ++qb) s_a[kb][qb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    scores_tile<HD, QB>(sk, qf, s_a, lane);
+    if (causal_wg || (NT == 1 && ragged)) mask_scores<QB>(s_a, klim, lane);
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const float m0 = tile_row_max<QB>(s_a, qb);      // exact first reference: every row has at least one finite score
         // can any score of this wave's rows exceed its reference by more than 2^kSafeLog2?  (1 % slack for the fp32
         // accumulation of the dot products and of the norms; a NaN compares as "yes")
-        if constexpr (BOUND)
-            need_max = need_max || __builtin_amdgcn_ballot_w64(!(qnorm[qs] * kmax_all * 1.01f - m0 <= kSafeLog2)) != 0;
+        need_max = need_max || __builtin_amdgcn_ballot_w64(!(qnorm[qb] * kmax_all * 1.01f - m0 <= kSafeLog2)) != 0;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            s_a[qs][0][v] -= m0;
-            s_a[qs][1][v] -= m0;
-            negm[qs][v] = -m0;
+        for (int e = 0; e < 4; ++e) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) s_a[kb][qb][e] -= m0;
+            negm[qb][e] = -m0;
         }
     }
-    bf16x8 kw[KWIN][2];
+    bf16x8 kw[KWIN][KB];
     preload_k<HD>(sk + TILE_BYTES, kw, lane);      // K(1) for step 0
 
     // step j: S(j+1) from K slot (j+1)%3, P(j) V(j) from V slot j%4, K(j+2) fragments preloaded from slot (j+2)%3.
@@ -512,9 +505,9 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         auto load_v = [&]() { issue(vbase, vpre, sv_addr, j + 3, v_fill); };                                    \
         if (!late_sync) { sync(); load_k(); }                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
-        int nvalid[QS];                                                                                         \
-        _Pragma("unroll") for (int qs = 0; qs < QS; ++qs) nvalid[qs] = klim[qs] - (j + 1) * BN;                 \
-        pipe_step<HD, QS, BOUND>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },               \
+        int nvalid[QB];                                                                                         \
+        _Pragma("unroll") for (int qb = 0; qb < QB; ++qb) nvalid[qb] = klim[qb] - (j + 1) * BN;                 \
+        pipe_step<HD, QB>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },               \
                           sk + ks_next * TILE_BYTES, sv + v_cur * TILE_BYTES, sk + k_next2 * TILE_BYTES, qf, kw, \
                           SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 >= NT), nvalid,   \
                           need_max);                                                                            \
@@ -531,24 +524,23 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
 #undef CDM_ATTN_STEP
     // no direct-to-LDS write may outlive the workgroup; after the barrier no wave reads the K / V rings any more and
     // each wave stages its output rows there, so that they leave as whole 2 * HD-byte rows (16 bytes per lane, 4 or 8 rows
-    // per store) instead of 8-byte pieces of 32 different rows
+    // per store) instead of 8-byte pieces of 16 different rows
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     constexpr int PITCH = HD * 2 + 16;
     static_assert((NW / 2) * 32 * QS * PITCH <= RING * TILE_BYTES, "staging area exceeds a ring");
     char* stage = (wave < NW / 2 ? sk : sv) + (wave % (NW / 2)) * (32 * QS * PITCH);     // half the waves per ring
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
-        const float l_tot = l_run[qs] + __shfl_xor(l_run[qs], 32, 64);
+    for (int qb = 0; qb < QB; ++qb) {
+        float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
+        l_tot += __shfl_xor(l_tot, 32, 64);
         const float inv = 1.0f / l_tot;
 #pragma unroll
-        for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint2 w;
-                w.x = pack_bf16x2(oacc[qs][t][4 * g + 0] * inv, oacc[qs][t][4 * g + 1] * inv);
-                w.y = pack_bf16x2(oacc[qs][t][4 * g + 2] * inv, oacc[qs][t][4 * g + 3] * inv);
-                *reinterpret_cast<uint2*>(stage + (qs * 32 + r32) * PITCH + (32 * t + 8 * g + 4 * kh) * 2) = w;
-            }
+        for (int hb = 0; hb < HB; ++hb) {
+            uint2 w;
+            w.x = pack_bf16x2(oacc[hb][qb][0] * inv, oacc[hb][qb][1] * inv);
+            w.y = pack_bf16x2(oacc[hb][qb][2] * inv, oacc[hb][qb][3] * inv);
+            *reinterpret_cast<uint2*>(stage + (qb * 16 + r16) * PITCH + (16 * hb + 4 * g4) * 2) = w;
+        }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
     constexpr int LPR = HD / 8, RPI = 64 / LPR;             // lanes per row, rows per store instruction
@@ -661,8 +653,12 @@ __global__ __launch_bounds__(256) void pack_kv_kernel(const bf16_t* __restrict__
         const int row = idx % HD, c = idx / HD;                            // channel row, key chunk
         uint32_t w[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-            w[e] = (uint32_t)tile[c * 8 + 2 * e][row] | ((uint32_t)tile[c * 8 + 2 * e + 1][row] << 16);
+        for (int e = 0; e < 4; ++e) {
+            // chunk c = 4 s + g lists keys 32 s + 4 g + {0..3}, 32 s + 16 + 4 g + {0..3}: the order in which a lane of the
+            // attention kernel holds its probabilities of the 32-key step s
+            const int key = 32 * (c >> 2) + 4 * (c & 3) + 16 * (e >> 1) + 2 * (e & 1);
+            w[e] = (uint32_t)tile[key][row] | ((uint32_t)tile[key + 1][row] << 16);
+        }
         *reinterpret_cast<uint4*>(vt + (c * HD + row) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
@@ -797,12 +793,12 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     // variant 0 = 32 query rows per wave (8 waves, two per SIMD), row maxima dropped where the norm bound allows;
     // cross-checks: 1 = 64 query rows per wave (4 waves), 2 = variant 0 with the row maxima always taken
     const int variant = cdm_get_variant(0);
-#define CDM_ATTN_LAUNCH(QS_, BOUND_, THREADS)                                                   \
-    if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_, BOUND_><<<grid, THREADS, 0, st>>>(p);  \
-    else attn_fwd_pipe_kernel<64, QS_, BOUND_><<<grid, THREADS, 0, st>>>(p)
-    if (variant == 1) { CDM_ATTN_LAUNCH(2, false, 256); }
-    else if (variant == 2) { CDM_ATTN_LAUNCH(1, false, 512); }
-    else { CDM_ATTN_LAUNCH(1, true, 512); }
+    p.always_max = variant == 2;
+#define CDM_ATTN_LAUNCH(QS_, THREADS)                                                   \
+    if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_><<<grid, THREADS, 0, st>>>(p);  \
+    else attn_fwd_pipe_kernel<64, QS_><<<grid, THREADS, 0, st>>>(p)
+    if (variant == 1) { CDM_ATTN_LAUNCH(2, 256); }
+    else { CDM_ATTN_LAUNCH(1, 512); }
 #undef CDM_ATTN_LAUNCH
     return cdm_check_launch("attn_fwd_packed");
 }
