@@ -115,6 +115,8 @@ def main():
     ap.add_argument("--attn-variant", type=int, default=0)
     ap.add_argument("--gemm-variant", type=int, default=0)
     ap.add_argument("--rope", default="in_attention", choices=["in_attention", "gemm_epilogue", "streaming"])
+    ap.add_argument("--no-fused-pack", action="store_true",
+                    help="K / V rows from the QKV GEMM and a re-tiling kernel instead of tile images from its epilogue")
     ap.add_argument("--graph", action="store_true",
                     help="record the forward into a HIP graph once and time replays (launch-bound shapes such as C0)")
     ap.add_argument("--residual", default="fp32", choices=["fp32", "bf16"],
@@ -152,10 +154,10 @@ def main():
         return bench_attention_only(cfg, args, dev)
     stack = DMStack(cfg, device=dev)
     stack.reset_parameters()
-    if args.rope != "in_attention":
+    if args.rope != "in_attention" or args.no_fused_pack:
         from cosmos_amd import DMAttnProcessor
         for blk in stack.blocks:
-            blk.attn.set_processor(DMAttnProcessor(rope=args.rope))
+            blk.attn.set_processor(DMAttnProcessor(rope=args.rope, fuse_kv_pack=not args.no_fused_pack))
     # the weights were drawn from a generator seeded with cfg.seed: the inputs take another stream (the same seed would
     # reproduce the weights' random numbers, i.e. token rows parallel to weight rows)
     g = torch.Generator(device=dev).manual_seed(cfg.seed + 1000)
@@ -233,7 +235,7 @@ def main():
         "config": {"workload": f"{cfg.name}: {cfg.n_blocks} DM blocks, d={cfg.d_model}, {cfg.n_heads}x{cfg.head_dim} heads, "
                                f"SwiGLU {cfg.hidden}, {cfg.n_text} text + {cfg.grid[0]}x{cfg.grid[1]}x{cfg.grid[2]} video"
                                f" + {cfg.n_action} action = {cfg.n_tokens} tokens, batch 1",
-                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope,
+                   "n_tokens": cfg.n_tokens, "n_blocks": cfg.n_blocks, "attn_variant": args.attn_variant, "gemm_variant": args.gemm_variant, "rope": args.rope, "kv_pack": "separate kernel" if args.no_fused_pack or args.rope != "in_attention" else "qkv gemm epilogue",
                    "residual_stream": args.residual, "hip_graph": bool(args.graph)},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_pipe_kernel", "achieved": round(attn_tflops, 1), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(attn_tflops / peak, 4),

@@ -88,16 +88,19 @@ class DMAttnProcessor:
     attention over the joint sequence, per-branch output projection (optionally fused with the gated
     residual).
 
-    ``rope`` selects where mRoPE is applied: "in_attention" (default: in registers, to K while the attention
-    entry point re-tiles it and to Q when the attention kernel loads it - no extra pass over memory),
-    "gemm_epilogue" (on the fp32 accumulators of the QKV GEMM) or "streaming" (the in-place kernel after a plain
-    QKV GEMM).
+    ``rope`` selects where mRoPE is applied: "in_attention" (default: in registers, to K while it is re-tiled for
+    the attention kernel and to Q when that kernel loads it - no extra pass over memory), "gemm_epilogue" (on the
+    fp32 accumulators of the QKV GEMM) or "streaming" (the in-place kernel after a plain QKV GEMM).
+    ``fuse_kv_pack`` (with "in_attention"): the QKV GEMM writes K and V straight into the attention kernel's tile
+    images instead of rows that a second kernel re-tiles; taken where the layout allows it (head_dim 128, no
+    QK-RMSNorm, every token segment starting on a multiple of 64), the two-kernel form otherwise.
     """
 
-    def __init__(self, rope: str = "in_attention"):
+    def __init__(self, rope: str = "in_attention", fuse_kv_pack: bool = True):
         if rope not in ("in_attention", "gemm_epilogue", "streaming"):
             raise ValueError(f"unknown rope placement {rope!r}")
         self.rope = rope
+        self.fuse_kv_pack = bool(fuse_kv_pack)
 
     def __call__(self, attn: "DMAttention", hidden_states: torch.Tensor,
                  encoder_hidden_states: Optional[torch.Tensor] = None, attention_mask: Optional[torch.Tensor] = None,
@@ -149,6 +152,14 @@ class DMAttnProcessor:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
                          rope_cols=d + dkv, head_dim=attn.head_dim)
             ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
+        elif (self.rope == "in_attention" and self.fuse_kv_pack and qkn is None
+              and ops.qkv_pack_applies([(s0, ln) for (s0, ln, _, _) in modality_segments], attn.head_dim)):
+            if wsb is None:
+                wsb = torch.empty((ops.attn_workspace_bytes(n, attn.n_kv_heads, attn.head_dim),), dtype=torch.uint8,
+                                  device=x.device)
+            attn._qkv_pack(x, quant_scale, modality_segments, qkv, wsb, cos, sin)
+            ops.attention_packed(q, wsb, attn.n_heads, attn.head_dim, o, cos, sin, None, prefix, causal_prefix,
+                                 attn.n_kv_heads)
         else:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
             if self.rope == "streaming":
@@ -215,6 +226,18 @@ class _AttentionCore:
         _routed_linear(a, sa, self._weights(which), self._q.get(which) if self.fp8 else None, None, segments, out=out,
                        epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
                        head_dim=head_dim)
+
+    def _qkv_pack(self, a: torch.Tensor, sa: Optional[torch.Tensor], segments: Sequence[Segment], qkv: torch.Tensor,
+                  images: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+        """QKV projection with K (rotated) and V written as the attention kernel's tile images; Q into qkv[:, :d]."""
+        segl = [(s0, ln) for (s0, ln, _, _) in segments]
+        if self.fp8:
+            qw = self._q["qkv"]
+            ws, sws = [qw[b][0] for (_, _, b, _) in segments], [qw[b][1] for (_, _, b, _) in segments]
+        else:
+            ws, sws = [_data(self.qkv_weight[b]) for (_, _, b, _) in segments], None
+        ops.gemm_qkv_pack(a, sa if self.fp8 else None, ws, sws, segl, self.n_heads, self.n_kv_heads, self.head_dim,
+                          qkv[:, :self.d_model], images, cos, sin)
 
 
 def _data(t):

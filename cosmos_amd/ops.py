@@ -279,6 +279,58 @@ def grouped_gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wqs: Sequence[torch.Ten
     return out
 
 
+@_timed("gemm")
+def gemm_qkv_pack(a: torch.Tensor, sa: Optional[torch.Tensor], ws: Sequence[torch.Tensor],
+                  sws: Optional[Sequence[torch.Tensor]], segments: Sequence[Tuple[int, int]], n_heads: int,
+                  n_kv_heads: int, head_dim: int, q_out: torch.Tensor, workspace: torch.Tensor,
+                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None) -> None:
+    """Fused QKV projection: rows [start, start+len) of ``a`` use ws[g] = [d_q + 2 d_kv, K]; Q goes to ``q_out``
+    ([n, >= d_q] bf16 rows, not rotated), K (rotated with cos/sin when given) and V go straight into the attention
+    kernel's tile images in ``workspace`` (for ``attention_packed``).  e4m3 operands when ``sa`` / ``sws`` are given.
+    Raises where the fused form does not apply (``qkv_pack_applies`` tells beforehand)."""
+    lib = _lib.load()
+    M, K = a.shape
+    n_seg = len(segments)
+    ldw = ws[0].stride(0)
+    for w in ws:
+        if w.shape != ws[0].shape or w.stride(0) != ldw:
+            raise ValueError("all segment weights must share shape and row stride")
+    if ws[0].shape[0] != (n_heads + 2 * n_kv_heads) * head_dim:
+        raise ValueError("fused QKV weights must have (n_heads + 2 n_kv_heads) * head_dim rows")
+    PP = C.c_void_p * n_seg
+    I64 = C.c_int64 * n_seg
+    st, ln = I64(*[int(s) for s, _ in segments]), I64(*[int(l) for _, l in segments])
+    half = head_dim // 2
+    n = sum(int(l) for _, l in segments)
+    tail = (_f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half), _chk(workspace, "workspace", torch.uint8, 1),
+            workspace.numel(), _stream())
+    if sa is None:
+        wp = PP(*[_chk(w, "w", torch.bfloat16, 2) for w in ws])
+        rc = lib.cdm_grouped_gemm_qkv_pack_bf16(_chk(a, "a", torch.bfloat16, 2), a.stride(0), wp, ldw,
+                                                _chk(q_out, "q_out", torch.bfloat16, 2), q_out.stride(0), st, ln, n_seg, K,
+                                                n_heads, n_kv_heads, head_dim, *tail)
+        _lib.check(rc, "cdm_grouped_gemm_qkv_pack_bf16")
+    else:
+        N = ws[0].shape[0]
+        wp = PP(*[_chk(w, "wq", FP8_DTYPE, 2) for w in ws])
+        swp = PP(*[_f32vec(s, "sw", N) for s in sws])
+        rc = lib.cdm_grouped_gemm_qkv_pack_fp8(_chk(a, "aq", FP8_DTYPE, 2), a.stride(0), _f32vec(sa, "sa", M), wp, swp, ldw,
+                                               _chk(q_out, "q_out", torch.bfloat16, 2), q_out.stride(0), st, ln, n_seg, K,
+                                               n_heads, n_kv_heads, head_dim, *tail)
+        _lib.check(rc, "cdm_grouped_gemm_qkv_pack_fp8")
+
+
+def qkv_pack_applies(segments: Sequence[Tuple[int, int]], head_dim: int) -> bool:
+    """Whether ``gemm_qkv_pack`` accepts this token layout: head_dim 128, segments tiling [0, n) in order, each
+    starting on a multiple of 64 tokens."""
+    pos = 0
+    for s, l in segments:
+        if int(s) != pos or pos % 64:
+            return False
+        pos += int(l)
+    return head_dim == 128 and pos > 0
+
+
 # ----------------------------------------------------------------------------- RoPE / attention
 @_timed("rope")
 def mrope_qk_(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor, n_heads: int,

@@ -45,8 +45,9 @@ typedef enum cdm_epilogue {
     CDM_EPI_GATE_RESIDUAL = 2, /* C = R + gate[n] * (A W^T)            (gate may be null = 1) */
     CDM_EPI_ROPE_QK = 3,       /* C = A W^T with rotate-half RoPE applied to the columns
                                   below `rope_cols` (heads of width head_dim)            */
-    CDM_EPI_GATE_RESIDUAL_F32 = 4 /* CDM_EPI_GATE_RESIDUAL with C and R stored as fp32: the residual stream kept in
+    CDM_EPI_GATE_RESIDUAL_F32 = 4, /* CDM_EPI_GATE_RESIDUAL with C and R stored as fp32: the residual stream kept in
                                   fp32 (28 roundings of the stream to bf16 alone cost percent-level accuracy) */
+    CDM_EPI_QKV_PACK = 5       /* internal to cdm_grouped_gemm_qkv_pack_*: rejected by the general GEMM entry points */
 } cdm_epilogue;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -259,9 +260,34 @@ int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const
  * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default of either.
  *   "attn": 1 = 64 query rows per wave (four waves per workgroup), 2 = the default kernel with per-tile row maxima always
  *           taken (the default drops them where the norm bound of the scores allows);
- *   "gemm": 1 = two-stage pipeline with four waves and 32 x 32 MFMAs, 3 = five-slot ring with four waves and 32 x 32 MFMAs,
- *           instead of the five-slot ring with eight waves and 16 x 16 MFMAs. */
+ *   "gemm": 1 = two-stage pipeline with four waves and 32 x 32 MFMAs instead of the five-slot ring with eight waves and
+ *           16 x 16 MFMAs. */
 int32_t cdm_set_variant(const char* op, int32_t variant);
+
+/*
+ * Fused QKV projection of the shared attention (the three projections add_q_proj / add_k_proj / add_v_proj resp.
+ * to_q / to_k / to_v of transformers models/cosmos3_omni/modeling_cosmos3_omni.py:41-46, concatenated row-wise into
+ * W[g] = [d_q + 2 d_kv, K] per branch) whose K and V columns never reach memory as rows: each 64-token x 128-channel
+ * piece leaves the GEMM as the attention kernel's tile image - K rotated with cos/sin ([n_tokens, 64] fp32, may both
+ * be null) on the way, V transposed, the largest key norm of the tile recorded - what cdm_attn_pack_kv_bf16 would
+ * have produced from the K / V rows (V bit for bit; K is rotated from the fp32 accumulators here, from the rows
+ * rounded to bf16 there: one rounding less).  Q (columns [0, d_q)) is written to
+ * Q [n_tokens, ldq] as plain rows, NOT rotated: cdm_attn_fwd_packed_bf16 rotates it at load when given the tables.
+ * `workspace` (cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim) bytes, n_tokens = sum of seg_len) is then
+ * passed to cdm_attn_fwd_packed_bf16.  Restrictions: head_dim 128; no QK-RMSNorm (the norm precedes the rotation and
+ * needs the un-fused pack); the segments tile [0, n_tokens) in order and each starts on a multiple of 64 tokens
+ * (CDM_ERR_UNSUPPORTED otherwise - callers fall back to the GEMM + cdm_attn_pack_kv_bf16 pair).
+ */
+int32_t cdm_grouped_gemm_qkv_pack_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw, void* Q,
+                                       int64_t ldq, const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg,
+                                       int64_t K, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
+                                       const float* cos, const float* sin, void* workspace, int64_t workspace_bytes,
+                                       void* stream);
+int32_t cdm_grouped_gemm_qkv_pack_fp8(const void* Aq, int64_t lda, const float* sa, const void* const* Wq,
+                                      const float* const* sw, int64_t ldw, void* Q, int64_t ldq,
+                                      const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg, int64_t K,
+                                      int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, const float* cos,
+                                      const float* sin, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * Classifier-free-guidance combine fused with the scheduler's linear latent update - replaces, inside one

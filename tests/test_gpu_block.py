@@ -108,7 +108,9 @@ def test_mot_three_branch_block():
                 plist[b].copy_(plist[1])
     y3 = blk(x, temb, rot, [(0, 40, 0, True), (40, 64, 1, True), (104, 24, 2, True)])
     y1 = blk(x, temb, rot, [(0, cfg.n_tokens, 1, True)])
-    assert_close(y3, y1.float().cpu(), 0.99999, 2e-3, "equal weights == single branch")
+    # (the single segment takes the QKV GEMM that writes the K / V tile images itself and rotates K ahead of its one
+    # rounding; segments starting at 40 and 104 are not tile boundaries and take the GEMM + re-tiling pair)
+    assert_close(y3, y1.float().cpu(), 0.99999, 6e-3, "equal weights == single branch")
 
 
 @pytest.mark.parametrize("n_kv_heads", [None, 1])
