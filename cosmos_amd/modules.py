@@ -84,9 +84,8 @@ class Workspace:
 
 
 class DMAttnProcessor:
-    """Attention processor: per-branch QKV projection with mRoPE in the GEMM epilogue, ONE shared full
-    attention over the joint sequence, per-branch output projection (optionally fused with the gated
-    residual).
+    """Attention processor: per-branch QKV projection, rotate-half mRoPE, ONE shared full attention over the joint
+    sequence, per-branch output projection (optionally fused with the gated residual).
 
     ``rope`` selects where mRoPE is applied: "in_attention" (default: in registers, to K while it is re-tiled for
     the attention kernel and to Q when that kernel loads it - no extra pass over memory), "gemm_epilogue" (on the
