@@ -105,6 +105,20 @@ def test_bad_arguments_are_rejected_on_the_host():
                                         None) == _lib.ERR_BAD_SHAPE
     # the workspace holds K/V heads only
     assert lib.cdm_attn_workspace_bytes(100, 2, 64) * 3 == lib.cdm_attn_workspace_bytes(100, 6, 64)
+    # QKV projection with fused tile images: head_dim 128 only, segments tile the sequence on 64-token boundaries,
+    # the workspace must hold the images, and the general GEMM entry points refuse its epilogue code
+    W = (C.c_void_p * 2)(fake, fake)
+
+    def qp(starts, lens, hd=128, ws=1 << 24, H=2, Hkv=2):
+        st, ln = (C.c_int64 * len(starts))(*starts), (C.c_int64 * len(lens))(*lens)
+        return lib.cdm_grouped_gemm_qkv_pack_bf16(fake, 256, W, 256, fake, H * hd, st, ln, len(starts), 256, H, Hkv, hd, None, None,
+                                                  fake, ws, None)
+    assert qp([0], [100], hd=64) == _lib.ERR_UNSUPPORTED
+    assert qp([0, 100], [100, 28]) == _lib.ERR_UNSUPPORTED and "multiple of 64" in _lib.last_error()
+    assert qp([0, 128], [64, 64]) == _lib.ERR_UNSUPPORTED           # a gap between the segments
+    assert qp([0], [100], ws=1024) == _lib.ERR_BAD_ARG and "workspace" in _lib.last_error()
+    assert qp([0], [100], H=3, Hkv=2) == _lib.ERR_BAD_SHAPE
+    assert g(epi=5) == _lib.ERR_BAD_ARG and "qkv_pack" in _lib.last_error()
 
 
 def test_step_arguments_are_validated_on_the_host():
