@@ -649,9 +649,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < 32; ++i) {
             const int ni = i >> 2, mi = i & 3;
             if constexpr (FP8)
+                // literal zero scale operands select the unscaled instruction (v_mfma_f32_16x16x128_f8f6f4: block scale 1,
+                // no scale-load prefix in front of every MFMA)
                 acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(B[ni & 3], cur[mi], acc[mi][ni], 0 /*A: e4m3*/,
-                                                                               0 /*B: e4m3*/, 0, 0x7f7f7f7f /*scale 1*/, 0,
-                                                                               0x7f7f7f7f);
+                                                                               0 /*B: e4m3*/, 0, 0, 0, 0);
             else
                 acc[mi][ni] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B[ni & 3], cur[mi], acc[mi][ni], 0, 0, 0);
             if (!LAST) {
