@@ -55,9 +55,9 @@ SIGNATURES = {
                                     _P, _I64, _I32, _P]),
     "cdm_cfg_step_f32": (_I32, [_P, _P, _P, _F32, C.POINTER(_P), _I32, C.POINTER(_F32), C.POINTER(_P), _I32, _I64, _P]),
     "cdm_grouped_gemm_qkv_pack_bf16": (_I32, [_P, _I64, C.POINTER(_P), _I64, _P, _I64, C.POINTER(_I64), C.POINTER(_I64), _I32,
-                                              _I64, _I32, _I32, _I32, _P, _P, _P, _I64, _P]),
+                                              _I64, _I32, _I32, _I32, _P, _P, _P, _P, _I64, _P]),
     "cdm_grouped_gemm_qkv_pack_fp8": (_I32, [_P, _I64, _P, C.POINTER(_P), C.POINTER(_P), _I64, _P, _I64, C.POINTER(_I64),
-                                             C.POINTER(_I64), _I32, _I64, _I32, _I32, _I32, _P, _P, _P, _I64, _P]),
+                                             C.POINTER(_I64), _I32, _I64, _I32, _I32, _I32, _P, _P, _P, _P, _I64, _P]),
     "cdm_grouped_gemm_bf16": (_I32, [_P, _I64, C.POINTER(_P), _I64, C.POINTER(_P), _P, _I64, C.POINTER(_I64),
                                      C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P, _P, _I64,
                                      _I32, _P]),

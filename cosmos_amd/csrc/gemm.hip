@@ -41,6 +41,7 @@ struct GemmSeg {
     const void* W; const void* W2;
     const float* gate;
     const float* sw; const float* sw2;   // fp8 only
+    const float* knw;                    // QKV_PACK only: the segment's K-norm weight row [head_dim] fp32, or null
 };
 
 struct GemmParams {
@@ -56,6 +57,7 @@ struct GemmParams {
     // attention kernel's tile images (64 keys x 128 channels per K / V head), with the largest key norm of every tile
     char* kp; char* vp; float* kmax;
     int d_q, d_kv, n_key_tiles;
+    float k_eps;                         // epsilon of the per-head RMSNorm of K (segments with a weight row)
     int tiles_n, total_tiles, n_seg;
     GemmSeg seg[kMaxSeg];
 };
@@ -64,7 +66,7 @@ struct GemmParams {
 struct Tile {
     int m0, m_end, tn;
     const void* W; const void* W2;
-    const float* gate; const float* sw; const float* sw2;
+    const float* gate; const float* sw; const float* sw2; const float* knw;
 };
 
 // XCD-aware tile assignment: workgroup ids are dealt round-robin over the 8 XCDs, so ids are remapped to give each
@@ -98,7 +100,7 @@ __device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
     t.m_end = __builtin_amdgcn_readfirstlane(sg.m_end);
     t.tn = __builtin_amdgcn_readfirstlane(in_group / gsz);
     t.W = uniform_ptr(sg.W); t.W2 = uniform_ptr(sg.W2);
-    t.gate = uniform_ptr(sg.gate); t.sw = uniform_ptr(sg.sw); t.sw2 = uniform_ptr(sg.sw2);
+    t.gate = uniform_ptr(sg.gate); t.sw = uniform_ptr(sg.sw); t.sw2 = uniform_ptr(sg.sw2); t.knw = uniform_ptr(sg.knw);
     return true;
 }
 
@@ -337,6 +339,26 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
                 acc.set(rs, cs, 1, acc.get(rs, cs, 1) * (sr * w4.y));
                 acc.set(rs, cs, 2, acc.get(rs, cs, 2) * (sr * w4.z));
                 acc.set(rs, cs, 3, acc.get(rs, cs, 3) * (sr * w4.w));
+            }
+        }
+        if (EPI == CDM_EPI_QKV_PACK && region == 1 && t.knw != nullptr) {
+            // per-head RMSNorm of K on the fp32 accumulators, ahead of the rotation: the wave's 128 columns are one head,
+            // a key's channels are spread over the four quarter-waves (lanes r, r + 16, r + 32, r + 48 share the row)
+            float ss = 0.0f;
+#pragma unroll
+            for (int cs = 0; cs < CS; ++cs)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ss += acc.get(rs, cs, e) * acc.get(rs, cs, e);
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            const float rn = rsqrtf(ss * (1.0f / 128.0f) + p.k_eps);
+#pragma unroll
+            for (int cs = 0; cs < CS; ++cs) {
+                const float4 w4 = *reinterpret_cast<const float4*>(t.knw + ACC::col_local(cs, lane));
+                acc.set(rs, cs, 0, acc.get(rs, cs, 0) * (rn * w4.x));
+                acc.set(rs, cs, 1, acc.get(rs, cs, 1) * (rn * w4.y));
+                acc.set(rs, cs, 2, acc.get(rs, cs, 2) * (rn * w4.z));
+                acc.set(rs, cs, 3, acc.get(rs, cs, 3) * (rn * w4.w));
             }
         }
         if ((EPI == CDM_EPI_ROPE_QK || EPI == CDM_EPI_QKV_PACK) && rope) {
@@ -762,7 +784,7 @@ int32_t validate(const char* who, int esize, const void* A, int64_t lda, const v
 struct HostSeg {
     int64_t start, len;
     const void* W; const void* W2;
-    const float* gate; const float* sw; const float* sw2;
+    const float* gate; const float* sw; const float* sw2; const float* knw;
 };
 
 // Launches the segments kMaxSeg at a time (one grid per batch).  p holds everything that is common to the segments.
@@ -783,6 +805,7 @@ int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epi
             total += g.tiles_m * p.tiles_n;
             g.tile_end = total;
             g.W = segs[i].W; g.W2 = segs[i].W2; g.gate = segs[i].gate; g.sw = segs[i].sw; g.sw2 = segs[i].sw2;
+            g.knw = segs[i].knw;
         }
         if (ns == 0) break;
         p.n_seg = ns; p.total_tiles = total;
@@ -811,7 +834,8 @@ int32_t grouped(const char* who, const void* A, int64_t lda, const float* sa, co
                 int64_t ldw, const void* const* W2, const float* const* sw2, void* C, int64_t ldc,
                 const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg, int64_t N, int64_t K, int32_t epilogue,
                 const void* R, int64_t ldr, const float* const* gate, const float* cos, const float* sin,
-                int64_t rope_cols, int32_t head_dim, void* stream, const GemmParams* pack = nullptr) {
+                int64_t rope_cols, int32_t head_dim, void* stream, const GemmParams* pack = nullptr,
+                const float* k_norm_rows = nullptr) {
     constexpr int esize = FP8 ? 1 : 2;
     CDM_REQUIRE(A && W && C && seg_start && seg_len, CDM_ERR_BAD_ARG, "%s: null pointer", who);
     CDM_REQUIRE((epilogue == CDM_EPI_QKV_PACK) == (pack != nullptr), CDM_ERR_BAD_ARG,
@@ -840,7 +864,7 @@ int32_t grouped(const char* who, const void* A, int64_t lda, const float* sa, co
             CDM_REQUIRE(seg_start[g] >= segs[h].start + segs[h].len || seg_start[g] + seg_len[g] <= segs[h].start,
                         CDM_ERR_BAD_ARG, "%s: segments %d and %d overlap", who, h, g);
         segs[g] = HostSeg{seg_start[g], seg_len[g], W[g], W2 ? W2[g] : nullptr, gt, FP8 ? sw[g] : nullptr,
-                          (FP8 && sw2) ? sw2[g] : nullptr};
+                          (FP8 && sw2) ? sw2[g] : nullptr, k_norm_rows ? k_norm_rows + (int64_t)g * head_dim : nullptr};
         if (seg_start[g] + seg_len[g] > max_end) max_end = seg_start[g] + seg_len[g];
     }
     CDM_REQUIRE(max_end < (1ll << 31) - 512, CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
@@ -855,7 +879,7 @@ int32_t grouped(const char* who, const void* A, int64_t lda, const float* sa, co
     p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
     if (pack) {
         p.kp = pack->kp; p.vp = pack->vp; p.kmax = pack->kmax;
-        p.d_q = pack->d_q; p.d_kv = pack->d_kv; p.n_key_tiles = pack->n_key_tiles;
+        p.d_q = pack->d_q; p.d_kv = pack->d_kv; p.n_key_tiles = pack->n_key_tiles; p.k_eps = pack->k_eps;
     }
     return run<FP8>(p, segs, n_seg, N, epilogue, (hipStream_t)stream, who);
 }
@@ -865,7 +889,7 @@ template <bool FP8>
 int32_t qkv_pack(const char* who, const void* A, int64_t lda, const float* sa, const void* const* W, const float* const* sw,
                  int64_t ldw, void* Q, int64_t ldq, const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg,
                  int64_t K, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, const float* cos, const float* sin,
-                 void* workspace, int64_t workspace_bytes, void* stream) {
+                 const cdm_qk_norm* qk_norm, void* workspace, int64_t workspace_bytes, void* stream) {
     CDM_REQUIRE(seg_start && seg_len && workspace, CDM_ERR_BAD_ARG, "%s: null pointer", who);
     CDM_REQUIRE(head_dim == 128, CDM_ERR_UNSUPPORTED, "%s: head_dim=%d (the fused images need 128)", who, head_dim);
     CDM_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && n_heads <= 65535, CDM_ERR_BAD_SHAPE,
@@ -883,6 +907,17 @@ int32_t qkv_pack(const char* who, const void* A, int64_t lda, const float* sa, c
         n_tokens += seg_len[g];
     }
     CDM_REQUIRE(n_tokens <= 65535ll * 64, CDM_ERR_BAD_SHAPE, "%s: sizes out of range", who);
+    if (qk_norm != nullptr) {
+        // one weight row per GEMM segment: the norm's segments must be the GEMM's
+        CDM_REQUIRE(qk_norm->k_weight && cdm_aligned16(qk_norm->k_weight) && qk_norm->seg_end, CDM_ERR_BAD_ARG,
+                    "%s: qk_norm needs an aligned k_weight table and seg_end", who);
+        CDM_REQUIRE(qk_norm->eps > 0.0f, CDM_ERR_BAD_ARG, "%s: qk_norm eps must be positive", who);
+        CDM_REQUIRE(qk_norm->n_seg == n_seg, CDM_ERR_BAD_ARG, "%s: qk_norm has %d segments, the projection %d", who,
+                    qk_norm->n_seg, n_seg);
+        for (int g = 0; g < n_seg; ++g)
+            CDM_REQUIRE(qk_norm->seg_end[g] == seg_start[g] + seg_len[g] || (g == n_seg - 1 && qk_norm->seg_end[g] >= n_tokens),
+                        CDM_ERR_BAD_ARG, "%s: qk_norm segment %d does not end where the projection's does", who, g);
+    }
     const int64_t need = cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim);
     CDM_REQUIRE(workspace_bytes >= need, CDM_ERR_BAD_ARG, "%s: workspace of at least %lld bytes required", who, (long long)need);
     const int64_t d_q = (int64_t)n_heads * head_dim, d_kv = (int64_t)n_kv_heads * head_dim;
@@ -893,8 +928,10 @@ int32_t qkv_pack(const char* who, const void* A, int64_t lda, const float* sa, c
     GemmParams pack{};
     pack.kp = (char*)workspace; pack.vp = (char*)workspace + img; pack.kmax = (float*)((char*)workspace + 2 * img);
     pack.d_q = (int)d_q; pack.d_kv = (int)d_kv; pack.n_key_tiles = (int)n_key_tiles;
+    pack.k_eps = qk_norm ? qk_norm->eps : 0.0f;
     int32_t rc = grouped<FP8>(who, A, lda, sa, W, sw, ldw, nullptr, nullptr, Q, ldq, seg_start, seg_len, n_seg, d_q + 2 * d_kv, K,
-                              CDM_EPI_QKV_PACK, nullptr, 0, nullptr, cos, sin, d_q, head_dim, stream, &pack);
+                              CDM_EPI_QKV_PACK, nullptr, 0, nullptr, cos, sin, d_q, head_dim, stream, &pack,
+                              qk_norm ? qk_norm->k_weight : nullptr);
     return rc;
 }
 
@@ -903,20 +940,21 @@ int32_t qkv_pack(const char* who, const void* A, int64_t lda, const float* sa, c
 extern "C" int32_t cdm_grouped_gemm_qkv_pack_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw, void* Q,
                                                   int64_t ldq, const int64_t* seg_start, const int64_t* seg_len,
                                                   int32_t n_seg, int64_t K, int32_t n_heads, int32_t n_kv_heads,
-                                                  int32_t head_dim, const float* cos, const float* sin, void* workspace,
-                                                  int64_t workspace_bytes, void* stream) {
+                                                  int32_t head_dim, const float* cos, const float* sin,
+                                                  const cdm_qk_norm* qk_norm, void* workspace, int64_t workspace_bytes,
+                                                  void* stream) {
     return qkv_pack<false>("grouped_gemm_qkv_pack_bf16", A, lda, nullptr, W, nullptr, ldw, Q, ldq, seg_start, seg_len, n_seg,
-                           K, n_heads, n_kv_heads, head_dim, cos, sin, workspace, workspace_bytes, stream);
+                           K, n_heads, n_kv_heads, head_dim, cos, sin, qk_norm, workspace, workspace_bytes, stream);
 }
 
 extern "C" int32_t cdm_grouped_gemm_qkv_pack_fp8(const void* Aq, int64_t lda, const float* sa, const void* const* Wq,
                                                  const float* const* sw, int64_t ldw, void* Q, int64_t ldq,
                                                  const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg,
                                                  int64_t K, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
-                                                 const float* cos, const float* sin, void* workspace,
-                                                 int64_t workspace_bytes, void* stream) {
+                                                 const float* cos, const float* sin, const cdm_qk_norm* qk_norm,
+                                                 void* workspace, int64_t workspace_bytes, void* stream) {
     return qkv_pack<true>("grouped_gemm_qkv_pack_fp8", Aq, lda, sa, Wq, sw, ldw, Q, ldq, seg_start, seg_len, n_seg, K,
-                          n_heads, n_kv_heads, head_dim, cos, sin, workspace, workspace_bytes, stream);
+                          n_heads, n_kv_heads, head_dim, cos, sin, qk_norm, workspace, workspace_bytes, stream);
 }
 
 extern "C" int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int64_t ldw, const void* W2, void* C,

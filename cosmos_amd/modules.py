@@ -91,8 +91,8 @@ class DMAttnProcessor:
     the attention kernel and to Q when that kernel loads it - no extra pass over memory), "gemm_epilogue" (on the
     fp32 accumulators of the QKV GEMM) or "streaming" (the in-place kernel after a plain QKV GEMM).
     ``fuse_kv_pack`` (with "in_attention"): the QKV GEMM writes K and V straight into the attention kernel's tile
-    images instead of rows that a second kernel re-tiles; taken where the layout allows it (head_dim 128, no
-    QK-RMSNorm, every token segment starting on a multiple of 64), the two-kernel form otherwise.
+    images instead of rows that a second kernel re-tiles; taken where the layout allows it (head_dim 128, every
+    token segment starting on a multiple of 64), the two-kernel form otherwise.
     """
 
     def __init__(self, rope: str = "in_attention", fuse_kv_pack: bool = True):
@@ -151,13 +151,13 @@ class DMAttnProcessor:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="rope_qk", cos=cos, sin=sin,
                          rope_cols=d + dkv, head_dim=attn.head_dim)
             ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
-        elif (self.rope == "in_attention" and self.fuse_kv_pack and qkn is None
+        elif (self.rope == "in_attention" and self.fuse_kv_pack
               and ops.qkv_pack_applies([(s0, ln) for (s0, ln, _, _) in modality_segments], attn.head_dim)):
             if wsb is None:
                 wsb = torch.empty((ops.attn_workspace_bytes(n, attn.n_kv_heads, attn.head_dim),), dtype=torch.uint8,
                                   device=x.device)
-            attn._qkv_pack(x, quant_scale, modality_segments, qkv, wsb, cos, sin)
-            ops.attention_packed(q, wsb, attn.n_heads, attn.head_dim, o, cos, sin, None, prefix, causal_prefix,
+            attn._qkv_pack(x, quant_scale, modality_segments, qkv, wsb, cos, sin, qkn)
+            ops.attention_packed(q, wsb, attn.n_heads, attn.head_dim, o, cos, sin, qkn, prefix, causal_prefix,
                                  attn.n_kv_heads)
         else:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
@@ -227,8 +227,9 @@ class _AttentionCore:
                        head_dim=head_dim)
 
     def _qkv_pack(self, a: torch.Tensor, sa: Optional[torch.Tensor], segments: Sequence[Segment], qkv: torch.Tensor,
-                  images: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
-        """QKV projection with K (rotated) and V written as the attention kernel's tile images; Q into qkv[:, :d]."""
+                  images: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, qk_norm=None) -> None:
+        """QKV projection with K (normalised, rotated) and V written as the attention kernel's tile images; Q into
+        qkv[:, :d]."""
         segl = [(s0, ln) for (s0, ln, _, _) in segments]
         if self.fp8:
             qw = self._q["qkv"]
@@ -236,7 +237,7 @@ class _AttentionCore:
         else:
             ws, sws = [_data(self.qkv_weight[b]) for (_, _, b, _) in segments], None
         ops.gemm_qkv_pack(a, sa if self.fp8 else None, ws, sws, segl, self.n_heads, self.n_kv_heads, self.head_dim,
-                          qkv[:, :self.d_model], images, cos, sin)
+                          qkv[:, :self.d_model], images, cos, sin, qk_norm)
 
 
 def _data(t):

@@ -283,11 +283,13 @@ def grouped_gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wqs: Sequence[torch.Ten
 def gemm_qkv_pack(a: torch.Tensor, sa: Optional[torch.Tensor], ws: Sequence[torch.Tensor],
                   sws: Optional[Sequence[torch.Tensor]], segments: Sequence[Tuple[int, int]], n_heads: int,
                   n_kv_heads: int, head_dim: int, q_out: torch.Tensor, workspace: torch.Tensor,
-                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None) -> None:
+                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, qk_norm=None) -> None:
     """Fused QKV projection: rows [start, start+len) of ``a`` use ws[g] = [d_q + 2 d_kv, K]; Q goes to ``q_out``
-    ([n, >= d_q] bf16 rows, not rotated), K (rotated with cos/sin when given) and V go straight into the attention
-    kernel's tile images in ``workspace`` (for ``attention_packed``).  e4m3 operands when ``sa`` / ``sws`` are given.
-    Raises where the fused form does not apply (``qkv_pack_applies`` tells beforehand)."""
+    ([n, >= d_q] bf16 rows, neither normalised nor rotated), K (normalised per head with row g of ``qk_norm``'s K
+    weights when given, then rotated with cos/sin when given) and V go straight into the attention kernel's tile
+    images in ``workspace`` (for ``attention_packed``, which takes the same ``qk_norm`` for Q).  ``qk_norm`` =
+    (q_weight, k_weight, seg_ends, eps) with one segment per GEMM segment.  e4m3 operands when ``sa`` / ``sws`` are
+    given.  Raises where the fused form does not apply (``qkv_pack_applies`` tells beforehand)."""
     lib = _lib.load()
     M, K = a.shape
     n_seg = len(segments)
@@ -302,7 +304,8 @@ def gemm_qkv_pack(a: torch.Tensor, sa: Optional[torch.Tensor], ws: Sequence[torc
     st, ln = I64(*[int(s) for s, _ in segments]), I64(*[int(l) for _, l in segments])
     half = head_dim // 2
     n = sum(int(l) for _, l in segments)
-    tail = (_f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half), _chk(workspace, "workspace", torch.uint8, 1),
+    qn, _keep = _qk_norm_arg(qk_norm, head_dim)
+    tail = (_f32vec(cos, "cos", n * half), _f32vec(sin, "sin", n * half), qn, _chk(workspace, "workspace", torch.uint8, 1),
             workspace.numel(), _stream())
     if sa is None:
         wp = PP(*[_chk(w, "w", torch.bfloat16, 2) for w in ws])
@@ -322,7 +325,7 @@ def gemm_qkv_pack(a: torch.Tensor, sa: Optional[torch.Tensor], ws: Sequence[torc
 
 def qkv_pack_applies(segments: Sequence[Tuple[int, int]], head_dim: int) -> bool:
     """Whether ``gemm_qkv_pack`` accepts this token layout: head_dim 128, segments tiling [0, n) in order, each
-    starting on a multiple of 64 tokens."""
+    starting on a multiple of 64 tokens (a 64-key tile image is written by one wave from one weight set)."""
     pos = 0
     for s, l in segments:
         if int(s) != pos or pos % 64:

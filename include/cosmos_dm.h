@@ -274,20 +274,24 @@ int32_t cdm_set_variant(const char* op, int32_t variant);
  * rounded to bf16 there: one rounding less).  Q (columns [0, d_q)) is written to
  * Q [n_tokens, ldq] as plain rows, NOT rotated: cdm_attn_fwd_packed_bf16 rotates it at load when given the tables.
  * `workspace` (cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim) bytes, n_tokens = sum of seg_len) is then
- * passed to cdm_attn_fwd_packed_bf16.  Restrictions: head_dim 128; no QK-RMSNorm (the norm precedes the rotation and
- * needs the un-fused pack); the segments tile [0, n_tokens) in order and each starts on a multiple of 64 tokens
+ * passed to cdm_attn_fwd_packed_bf16.  qk_norm (optional): the per-head RMSNorm of K (norm_k / norm_added_k) is applied
+ * to the fp32 accumulators ahead of the rotation, segment g of the projection using row g of qk_norm->k_weight
+ * (qk_norm->n_seg = n_seg, qk_norm->seg_end[g] = seg_start[g] + seg_len[g]); the Q rows leave un-normalised -
+ * cdm_attn_fwd_packed_bf16 normalises and rotates them at load when given the same descriptor.
+ * Restrictions: head_dim 128; the segments tile [0, n_tokens) in order and each starts on a multiple of 64 tokens
  * (CDM_ERR_UNSUPPORTED otherwise - callers fall back to the GEMM + cdm_attn_pack_kv_bf16 pair).
  */
 int32_t cdm_grouped_gemm_qkv_pack_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw, void* Q,
                                        int64_t ldq, const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg,
                                        int64_t K, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
-                                       const float* cos, const float* sin, void* workspace, int64_t workspace_bytes,
-                                       void* stream);
+                                       const float* cos, const float* sin, const cdm_qk_norm* qk_norm, void* workspace,
+                                       int64_t workspace_bytes, void* stream);
 int32_t cdm_grouped_gemm_qkv_pack_fp8(const void* Aq, int64_t lda, const float* sa, const void* const* Wq,
                                       const float* const* sw, int64_t ldw, void* Q, int64_t ldq,
                                       const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg, int64_t K,
                                       int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, const float* cos,
-                                      const float* sin, void* workspace, int64_t workspace_bytes, void* stream);
+                                      const float* sin, const cdm_qk_norm* qk_norm, void* workspace,
+                                      int64_t workspace_bytes, void* stream);
 
 /*
  * Classifier-free-guidance combine fused with the scheduler's linear latent update - replaces, inside one

@@ -109,15 +109,24 @@ def test_bad_arguments_are_rejected_on_the_host():
     # the workspace must hold the images, and the general GEMM entry points refuse its epilogue code
     W = (C.c_void_p * 2)(fake, fake)
 
-    def qp(starts, lens, hd=128, ws=1 << 24, H=2, Hkv=2):
+    def qp(starts, lens, hd=128, ws=1 << 24, H=2, Hkv=2, qkn=None):
         st, ln = (C.c_int64 * len(starts))(*starts), (C.c_int64 * len(lens))(*lens)
         return lib.cdm_grouped_gemm_qkv_pack_bf16(fake, 256, W, 256, fake, H * hd, st, ln, len(starts), 256, H, Hkv, hd, None, None,
-                                                  fake, ws, None)
+                                                  qkn, fake, ws, None)
     assert qp([0], [100], hd=64) == _lib.ERR_UNSUPPORTED
     assert qp([0, 100], [100, 28]) == _lib.ERR_UNSUPPORTED and "multiple of 64" in _lib.last_error()
     assert qp([0, 128], [64, 64]) == _lib.ERR_UNSUPPORTED           # a gap between the segments
     assert qp([0], [100], ws=1024) == _lib.ERR_BAD_ARG and "workspace" in _lib.last_error()
     assert qp([0], [100], H=3, Hkv=2) == _lib.ERR_BAD_SHAPE
+    # the K-norm descriptor must have the projection's segments
+    e2 = (C.c_int64 * 2)(64, 128)
+    qn2 = _lib.QkNorm(fake, fake, e2, 2, 1e-6)
+    assert qp([0], [128], qkn=C.addressof(qn2)) == _lib.ERR_BAD_ARG and "segments" in _lib.last_error()
+    e1 = (C.c_int64 * 1)(100)
+    qn1 = _lib.QkNorm(fake, fake, e1, 1, 1e-6)
+    assert qp([0], [128], qkn=C.addressof(qn1)) == _lib.ERR_BAD_ARG and "does not end" in _lib.last_error()
+    qn0 = _lib.QkNorm(fake, fake, e1, 1, 0.0)
+    assert qp([0], [100], qkn=C.addressof(qn0)) == _lib.ERR_BAD_ARG and "eps" in _lib.last_error()
     assert g(epi=5) == _lib.ERR_BAD_ARG and "qkv_pack" in _lib.last_error()
 
 

@@ -252,13 +252,17 @@ def test_gemm_gate_residual_fp32_stream(M, N, K, gated, fp8, variant, request):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("n,H,Hkv,K,rope,split", [(256, 2, 2, 256, False, 0), (1000, 4, 2, 512, True, 0), (800, 2, 1, 256, True, 320),
-                                                 (4100, 3, 3, 256, False, 1024), (64, 1, 1, 256, True, 0)])
-def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, fp8):
+@pytest.mark.parametrize("n,H,Hkv,K,rope,split,qkn", [(256, 2, 2, 256, False, 0, False), (1000, 4, 2, 512, True, 0, False),
+                                                     (800, 2, 1, 256, True, 320, False), (4100, 3, 3, 256, False, 1024, False),
+                                                     (64, 1, 1, 256, True, 0, False), (1000, 4, 2, 512, True, 0, True),
+                                                     (800, 2, 1, 256, True, 320, True), (300, 2, 2, 256, False, 128, True)])
+def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, qkn, fp8):
     """The QKV GEMM that writes K and V as the attention kernel's tile images, against the plain GEMM followed by the
-    re-tiling kernel: same Q rows, same V image and (without rotation) the same K image bit for bit, the same key-norm bounds to fp32 rounding;
-    with rotation K carries one rounding less, so the images agree to a bf16 ulp and the attention outputs to 1e-2.
-    Ragged last tiles (1000, 800, 4100 tokens), grouped K / V heads, two weight sets split on a tile boundary."""
+    re-tiling kernel: same Q rows, same V image and (without rotation or norm) the same K image bit for bit, the same
+    key-norm bounds to fp32 rounding; with rotation or the per-head RMSNorm K carries one rounding less (both act on the
+    fp32 accumulators), so the images agree to a bf16 ulp and the attention outputs to 1e-2.
+    Ragged last tiles (1000, 800, 4100, 300 tokens), grouped K / V heads, two weight sets (and two norm weight rows)
+    split on a tile boundary; with the norm the attention output is also checked against the oracle."""
     hd = 128
     g = gen(n + 7 * H + K)
     d, dkv = H * hd, Hkv * hd
@@ -267,6 +271,11 @@ def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, fp8):
     ws = [rand_bf16((d + 2 * dkv, K), g, 0.05)[0] for _ in segs]
     pos, _ = rotary.build_positions(0, (1, 1, n))
     cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48), device=dev()) if rope else (None, None)
+    norm = None
+    if qkn:
+        qw = 1.0 + 0.3 * torch.randn(len(segs), hd, generator=g)
+        kw = 1.0 + 0.3 * torch.randn(len(segs), hd, generator=g)
+        norm = (qw.to(dev()), kw.to(dev()), [s0 + ln for s0, ln in segs], 1e-6)
     if fp8:
         aq, sa = ops.quant_rows(a)
         wq = [ops.quant_rows(w) for w in ws]
@@ -275,28 +284,39 @@ def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, fp8):
         qkv = ops.grouped_gemm(a, ws, segs)
     q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
     nbytes = ops.attn_workspace_bytes(n, Hkv, hd)
-    img_ref = ops.attention_pack_kv(k, v, Hkv, hd, torch.zeros(nbytes, dtype=torch.uint8, device=dev()), cos, sin)
+    img_ref = ops.attention_pack_kv(k, v, Hkv, hd, torch.zeros(nbytes, dtype=torch.uint8, device=dev()), cos, sin, norm)
     img = torch.full((nbytes,), 0x5a, dtype=torch.uint8, device=dev())
     q_out = torch.zeros((n, d), dtype=torch.bfloat16, device=dev())
     if fp8:
-        ops.gemm_qkv_pack(aq, sa, [w for w, _ in wq], [s for _, s in wq], segs, H, Hkv, hd, q_out, img, cos, sin)
+        ops.gemm_qkv_pack(aq, sa, [w for w, _ in wq], [s for _, s in wq], segs, H, Hkv, hd, q_out, img, cos, sin, norm)
     else:
-        ops.gemm_qkv_pack(a, None, ws, None, segs, H, Hkv, hd, q_out, img, cos, sin)
+        ops.gemm_qkv_pack(a, None, ws, None, segs, H, Hkv, hd, q_out, img, cos, sin, norm)
     assert torch.equal(q_out, q)
     one = (n + 63) // 64 * 64 * dkv * 2
     assert torch.equal(img[one:2 * one], img_ref[one:2 * one]), "V image"
     n_tiles = (n + 63) // 64
     km, km_ref = img[2 * one:2 * one + 4 * Hkv * n_tiles].view(torch.float32), img_ref[2 * one:2 * one + 4 * Hkv * n_tiles].view(torch.float32)
-    if not rope:
+    if not rope and not qkn:
         assert torch.equal(img[:one], img_ref[:one]), "K image"
         assert torch.allclose(km, km_ref, rtol=1e-5), "key-norm bounds (the two kernels sum the squares in different orders)"
     else:
         kf, kr = img[:one].view(torch.bfloat16).float(), img_ref[:one].view(torch.bfloat16).float()
-        assert float((kf - kr).abs().max()) <= 2.0 ** -7 * float(kr.abs().max())
+        assert float((kf - kr).abs().max()) <= (2.0 ** -6 if qkn else 2.0 ** -7) * float(kr.abs().max())
         assert torch.allclose(km, km_ref, rtol=1e-2)
-    o = ops.attention_packed(q_out, img, H, hd, None, cos, sin, None, None, 0, Hkv)
-    o_ref = ops.attention_packed(q, img_ref, H, hd, None, cos, sin, None, None, 0, Hkv)
-    assert_close(o, o_ref, 0.9999, 1e-2, f"attention on fused images n={n} fp8={fp8}")
+    o = ops.attention_packed(q_out, img, H, hd, None, cos, sin, norm, None, 0, Hkv)
+    o_ref = ops.attention_packed(q, img_ref, H, hd, None, cos, sin, norm, None, 0, Hkv)
+    assert_close(o, o_ref, 0.9999, 1e-2, f"attention on fused images n={n} fp8={fp8} qkn={qkn}")
+    if qkn:      # against the oracle, from the projected rows the kernels saw (bf16 Q / K / V of the plain GEMM)
+        qr, kr_, vr = q.float().cpu().view(n, H, hd), k.float().cpu().view(n, Hkv, hd), v.float().cpu().view(n, Hkv, hd)
+        qn_, kn_ = torch.empty_like(qr), torch.empty_like(kr_)
+        for i, (s0, ln) in enumerate(segs):
+            qn_[s0:s0 + ln] = O.rms_norm(qr[s0:s0 + ln], qw[i], 1e-6)
+            kn_[s0:s0 + ln] = O.rms_norm(kr_[s0:s0 + ln], kw[i], 1e-6)
+        if rope:
+            qn_, kn_ = O.apply_mrope(qn_, cos.cpu(), sin.cpu()), O.apply_mrope(kn_, cos.cpu(), sin.cpu())
+        rep = H // Hkv
+        want = O.attention(qn_, kn_.repeat_interleave(rep, dim=1), vr.repeat_interleave(rep, dim=1))
+        assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"fused images with K-norm vs oracle n={n} fp8={fp8}")
     # layouts the fused form does not take are refused, not mis-tiled
     if n > 100:
         with pytest.raises(RuntimeError):
