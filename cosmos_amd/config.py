@@ -43,7 +43,8 @@ class DMConfig:
 
     def gemm_flops_per_block(self) -> float:
         n, d, h = self.n_tokens, self.d_model, self.hidden
-        return 8.0 * n * d * d + 6.0 * n * d * h
+        d_kv = self.kv_heads * self.head_dim          # = d unless K / V heads are grouped
+        return 2.0 * n * d * (2 * d + 2 * d_kv) + 6.0 * n * d * h
 
     def attn_flops_per_block(self) -> float:
         return 4.0 * float(self.n_tokens) ** 2 * self.d_model
