@@ -1,4 +1,5 @@
-// Library-wide host services: version, thread-local error text, device probe, variant knobs.
+// Library-wide host services: version, thread-local error text, device probe (and, in the cross-check build only, the
+// knob that selects a superseded kernel).
 #include <atomic>
 #include <mutex>
 #include <stdarg.h>
@@ -8,7 +9,9 @@
 
 namespace {
 thread_local char g_err[512] = "";
+#ifdef CDM_CROSSCHECK
 std::atomic<int> g_variant[2] = {{0}, {0}};
+#endif
 std::once_flag g_dev_once;
 int g_dev_count = 0;
 
@@ -35,7 +38,9 @@ int32_t cdm_require_device(void) {
     return CDM_OK;
 }
 
+#ifdef CDM_CROSSCHECK
 int32_t cdm_get_variant(int which) { return g_variant[which].load(std::memory_order_relaxed); }
+#endif
 
 #ifndef CDM_SOURCE_HASH
 #define CDM_SOURCE_HASH "unknown"
@@ -54,6 +59,7 @@ extern "C" int32_t cdm_device_count(void) {
     return g_dev_count;
 }
 
+#ifdef CDM_CROSSCHECK
 extern "C" int32_t cdm_set_variant(const char* op, int32_t variant) {
     CDM_REQUIRE(op, CDM_ERR_BAD_ARG, "set_variant: null op");
     int which = -1;
@@ -63,3 +69,4 @@ extern "C" int32_t cdm_set_variant(const char* op, int32_t variant) {
     CDM_REQUIRE(variant >= 0 && variant < 64, CDM_ERR_BAD_ARG, "set_variant: variant %d out of range", variant);
     return g_variant[which].exchange(variant);
 }
+#endif

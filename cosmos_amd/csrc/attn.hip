@@ -793,14 +793,17 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     dim3 grid((unsigned)nwg);
     hipStream_t st = (hipStream_t)stream;
     // variant 0 = 32 query rows per wave (8 waves, two per SIMD), row maxima dropped where the norm bound allows;
-    // cross-checks: 1 = 64 query rows per wave (4 waves), 2 = variant 0 with the row maxima always taken
+    // cross-check build only: 1 = 64 query rows per wave (4 waves), 2 = variant 0 with the row maxima always taken
     const int variant = cdm_get_variant(0);
     p.always_max = variant == 2;
 #define CDM_ATTN_LAUNCH(QS_, THREADS)                                                   \
     if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_><<<grid, THREADS, 0, st>>>(p);  \
     else attn_fwd_pipe_kernel<64, QS_><<<grid, THREADS, 0, st>>>(p)
+#ifdef CDM_CROSSCHECK
     if (variant == 1) { CDM_ATTN_LAUNCH(2, 256); }
-    else { CDM_ATTN_LAUNCH(1, 512); }
+    else
+#endif
+    { CDM_ATTN_LAUNCH(1, 512); }
 #undef CDM_ATTN_LAUNCH
     return cdm_check_launch("attn_fwd_packed");
 }
@@ -874,7 +877,15 @@ int32_t static_scratch(void** out) {
 
 }  // namespace
 
-extern "C" int64_t cdm_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+// Also the set-up call: with a device visible it resolves the array's address on the current device, so that a caller
+// which records cdm_attn_fwd_static_bf16 into a graph can have that done outside the capture.
+extern "C" int64_t cdm_attn_static_scratch_bytes(void) {
+    if (cdm_device_count() > 0) {
+        void* ws = nullptr;
+        (void)static_scratch(&ws);      // a failure is reported by the entry point itself
+    }
+    return kStaticScratchBytes;
+}
 
 extern "C" int32_t cdm_attn_fwd_static_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                                             int64_t ldv, const float* cos, const float* sin, void* o, int64_t ldo,

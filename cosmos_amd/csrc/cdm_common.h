@@ -37,7 +37,13 @@ static inline int32_t cdm_check_launch(const char* what) {
 }
 
 int32_t cdm_require_device(void);           // CDM_OK or CDM_ERR_NO_DEVICE (sets the message)
-int32_t cdm_get_variant(int which);         // 0 = attn, 1 = gemm
+// Kernel variant selected for an operator (0 = attn, 1 = gemm).  Only the cross-check build (-DCDM_CROSSCHECK) carries
+// the superseded kernels and the knob that selects them; the product library always runs the default kernels.
+#ifdef CDM_CROSSCHECK
+int32_t cdm_get_variant(int which);
+#else
+static inline int32_t cdm_get_variant(int) { return 0; }
+#endif
 
 // -------------------------------------------------------------- device side
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }

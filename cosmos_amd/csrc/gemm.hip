@@ -111,6 +111,7 @@ __device__ __forceinline__ bf16x8 lds_frag(const char* tile, int row, int chunk)
     return *reinterpret_cast<const bf16x8*>(tile + row * (BK * 2) + ((chunk ^ swz(row)) << 4));
 }
 
+#ifdef CDM_CROSSCHECK      // the two-stage pipeline on 32 x 32 MFMAs: main loop pieces
 template <bool FP8>
 __device__ __forceinline__ void compute_stage(const char* sa, const char* sb, f32x16 (&acc)[4][4], int wm, int wn,
                                               int lane) {
@@ -172,6 +173,8 @@ __device__ __forceinline__ void issue_loads(const char* abase, const char* wbase
     }
 }
 
+#endif
+
 // silu(g) = g / (1 + e^-g) with the hardware reciprocal (1 ulp) instead of an IEEE division: the result is rounded to
 // bf16 anyway, and a correctly rounded division is ten instructions per output value of a 128 x 64 result per wave
 __device__ __forceinline__ float silu_f(float g) {
@@ -217,6 +220,7 @@ __device__ __forceinline__ void copy_out(const GemmParams& p, const Tile& t, con
 
 // Views of a wave's accumulators: where in the wave's ROWS x 128 piece of the tile a lane's quads (four consecutive
 // columns of one row) sit.  RS row slots x CS column slots per lane; column slot cs + CS / 2 is 64 columns right of cs.
+#ifdef CDM_CROSSCHECK
 template <int MI>
 struct Acc32 {      // MI x 4 blocks of 32 x 32 (v_mfma_*_32x32x*): lane = row % 32 + 32 kh, quads at columns 8 g + 4 kh
     f32x16 (&v)[MI][4];
@@ -226,6 +230,7 @@ struct Acc32 {      // MI x 4 blocks of 32 x 32 (v_mfma_*_32x32x*): lane = row %
     __device__ __forceinline__ float get(int rs, int cs, int e) const { return v[rs][cs >> 2][4 * (cs & 3) + e]; }
     __device__ __forceinline__ void set(int rs, int cs, int e, float x) { v[rs][cs >> 2][4 * (cs & 3) + e] = x; }
 };
+#endif
 template <int MI>
 struct Acc16 {      // MI x 8 blocks of 16 x 16 (v_mfma_*_16x16x*): lane = row % 16 + 16 q, one quad per block at column 4 q
     f32x4 (&v)[MI][8];
@@ -463,6 +468,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
     if (stage) copy_out<128, 2, ROWS>(p, t, stage, row0, colw, lane);
 }
 
+#ifdef CDM_CROSSCHECK
 template <int EPI, bool FP8>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(1024))) char sa0[kTileBytes];
@@ -535,6 +541,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     epilogue<EPI, FP8>(p, tile, Acc32<4>{acc}, m0 + wm * 128, n0, wn, lane, nullptr);
 }
+#endif
 
 // ---------------------------------------------------------------------------------------------
 // Ring pipeline (default): 256 x 256 tile, EIGHT waves (two per SIMD), 16 x 16 MFMAs, 128-byte tile rows (k-tiles of
@@ -792,8 +799,10 @@ template <bool FP8>
 int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epilogue, hipStream_t st, const char* who) {
     const int tile_n = epilogue == CDM_EPI_SWIGLU ? BN / 2 : BN;
     p.tiles_n = (int)((N + tile_n - 1) / tile_n);
-    // variant 0 = ring pipeline with eight waves and 16 x 16 MFMAs; 1 = two-stage pipeline, four waves, 32 x 32 MFMAs
+    // variant 0 = ring pipeline with eight waves and 16 x 16 MFMAs; 1 (cross-check build only) = two-stage pipeline, four
+    // waves, 32 x 32 MFMAs
     const bool ring = cdm_get_variant(1) != 1;
+    (void)ring;
     int i = 0;
     while (i < n_seg) {
         int ns = 0, total = 0;
@@ -810,9 +819,13 @@ int32_t run(GemmParams p, const HostSeg* segs, int n_seg, int64_t N, int32_t epi
         if (ns == 0) break;
         p.n_seg = ns; p.total_tiles = total;
         const int grid = ((total + 7) / 8) * 8;
+#ifdef CDM_CROSSCHECK
 #define CDM_LAUNCH(E)                                                         \
     if (ring) gemm_ring_kernel<E, FP8><<<grid, 512, 0, st>>>(p);            \
     else gemm_kernel<E, FP8><<<grid, kThreads, 0, st>>>(p)
+#else
+#define CDM_LAUNCH(E) gemm_ring_kernel<E, FP8><<<grid, 512, 0, st>>>(p)
+#endif
         switch (epilogue) {
             case CDM_EPI_NONE: CDM_LAUNCH(CDM_EPI_NONE); break;
             case CDM_EPI_SWIGLU: CDM_LAUNCH(CDM_EPI_SWIGLU); break;

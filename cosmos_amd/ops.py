@@ -87,11 +87,9 @@ def time_ops(enable: bool):
 
 
 def set_variant(op: str, variant: int) -> int:
-    lib = _lib.load()
-    prev = lib.cdm_set_variant(op.encode(), int(variant))
-    if prev < 0:
-        raise RuntimeError(f"set_variant failed: {_lib.last_error()}")
-    return prev
+    """Cross-check aid (tests, measurements): run ``op`` ("attn" / "gemm") on a superseded kernel of the cross-check
+    build; 0 = back to the product library's kernel.  Returns the previous selection."""
+    return _lib.set_variant(op, variant)
 
 
 # ----------------------------------------------------------------------------- norm / quant

@@ -219,7 +219,9 @@ int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, c
  * nothing.  Shapes whose images (cdm_attn_workspace_bytes) exceed that size are rejected with CDM_ERR_BAD_SHAPE.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
  * threads) race; calls on one stream are ordered and need no clearing in between (every call rewrites all
- * tiles it reads, padding included).
+ * tiles it reads, padding included).  The array's address is looked up once per device, by the first call on that
+ * device or by cdm_attn_static_scratch_bytes(): before recording the entry point into a graph, call either outside the
+ * capture with that device current.
  */
 #define CDM_ATTN_STATIC_SCRATCH_BYTES (32ll << 20)
 int64_t cdm_attn_static_scratch_bytes(void);
@@ -256,13 +258,17 @@ int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const
                              const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
                              void* stream);
 
-/* Knob for tests and measurements, process-wide (not per thread or stream): selects a kernel variant by name; returns the
- * previous value, or a negative status for an unknown name/value.  Default 0 = the tuned default of either.
+/* Exported by the cross-check build only (libcosmos_dm_hip_crosscheck.so, compiled with -DCDM_CROSSCHECK), which the
+ * parity tests load to compare the default kernels with their predecessors; the product library has no such state.
+ * Process-wide (not per thread or stream): selects a kernel variant by name; returns the previous value, or a negative
+ * status for an unknown name/value.  Default 0 = the kernels of the product library.
  *   "attn": 1 = 64 query rows per wave (four waves per workgroup), 2 = the default kernel with per-tile row maxima always
  *           taken (the default drops them where the norm bound of the scores allows);
  *   "gemm": 1 = two-stage pipeline with four waves and 32 x 32 MFMAs instead of the five-slot ring with eight waves and
  *           16 x 16 MFMAs. */
+#ifdef CDM_CROSSCHECK
 int32_t cdm_set_variant(const char* op, int32_t variant);
+#endif
 
 /*
  * Fused QKV projection of the shared attention (the three projections add_q_proj / add_k_proj / add_v_proj resp.

@@ -13,10 +13,14 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HAS_GPU = torch.cuda.is_available()
 
 
-def header_functions():
+def header_functions(crosscheck=False):
+    """Function names the header declares for the product library (or, crosscheck=True, inside its
+    ``#ifdef CDM_CROSSCHECK`` sections: the extra exports of the cross-check build)."""
     text = open(os.path.join(ROOT, "include", "cosmos_dm.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(cdm_[a-z0-9_]+)\s*\(", text)))
+    guarded = "".join(re.findall(r"#ifdef CDM_CROSSCHECK(.*?)#endif", text, flags=re.S))
+    plain = re.sub(r"#ifdef CDM_CROSSCHECK.*?#endif", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cdm_[a-z0-9_]+)\s*\(", guarded if crosscheck else plain)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -26,6 +30,15 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/cosmos_dm.h but not exported"
     assert set(names) == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
+    # the product library carries no process-wide knob; the cross-check build exports it on top of the same ABI
+    extra = header_functions(crosscheck=True)
+    assert extra == sorted(_lib.CROSSCHECK_SIGNATURES) == ["cdm_set_variant"]
+    assert not hasattr(lib, "cdm_set_variant")
+    xlib = _lib.load_crosscheck()
+    for n in names + extra:
+        assert hasattr(xlib, n), f"{n} missing from the cross-check build"
+    assert xlib.cdm_set_variant(b"nope", 0) == _lib.ERR_BAD_ARG
+    assert xlib.cdm_source_hash() == lib.cdm_source_hash()
     assert lib.cdm_version() >= 100
     # two tile images of 128 padded tokens x 2 heads x 64 channels (bf16) + one fp32 key-norm bound per (head, tile)
     assert lib.cdm_attn_workspace_bytes(100, 2, 64) == 2 * 128 * 2 * 64 * 2 + 2 * 2 * 4
@@ -73,7 +86,6 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_fwd_static_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 0, 1, 1, 64, None, 0, None) == _lib.OK
     assert lib.cdm_mrope_qk_bf16(fake, 64, None, 0, fake, fake, 4, 1, 32, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_quant_rows_e4m3(fake, 128, fake, fake, 4, 100, None) == _lib.ERR_BAD_SHAPE
-    assert lib.cdm_set_variant(b"nope", 0) == _lib.ERR_BAD_ARG
     # empty inputs are accepted without work
     assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, fake, None, fake, 64, 16, 1, 1, 64, fake, 1 << 20, None, 0, None) == _lib.ERR_BAD_ARG   # cos without sin
     assert lib.cdm_attn_fwd_bf16(fake, 64, fake, 64, fake, 64, None, None, fake, 64, 0, 1, 1, 64, None, 0, None, 0, None) == _lib.OK

@@ -44,6 +44,41 @@ def test_first_order_step_is_the_euler_flow_step():
         assert np.allclose(y, want, atol=1e-12)
 
 
+def test_step_that_starts_at_sigma_one_is_the_limit_of_steps_that_start_just_below():
+    """A step from sigma = 1 has lambda = -inf and an infinite h; there both the oracle and the product's scheduler
+    take B(h) = e^h - 1 -> -1 whatever the solver type (B(h) = h, "bh1", has no limit).  Pinned from the other side:
+    the generic finite-h "bh2" code path at sigma_0 = 1 - eps must converge to the special case as eps -> 0, for
+    the predictor and the corrector; the corrector of order 1 must equal its closed form
+    sigma_t x + (1 - sigma_t) (m_0 + m_t) / 2; and a constant data prediction must be integrated exactly,
+    x_t = sigma_t x + (1 - sigma_t) c.  "bh1" on that one step is therefore "bh2": a recorded deviation."""
+    from cosmos_amd.sampler import _Update
+    rng = np.random.default_rng(5)
+    x, m0, mt = rng.standard_normal(6), rng.standard_normal(6), rng.standard_normal(6)
+    st = 0.83
+    at_one_p = U.unip_update(x, [m0], [1.0], st, 1)
+    at_one_c = U.unic_update(x, [m0], [1.0], mt, st, 1)
+    assert np.allclose(at_one_c, st * x + (1 - st) * 0.5 * (m0 + mt), atol=1e-13)
+    assert np.allclose(U.unic_update(x, [m0], [1.0], m0, st, 1), st * x + (1 - st) * m0, atol=1e-13)
+    for solver_type in ("bh1", "bh2"):
+        assert np.allclose(U.unic_update(x, [m0], [1.0], mt, st, 1, solver_type), at_one_c, atol=1e-13)
+    prev_p = prev_c = None
+    for eps in (1e-3, 1e-5, 1e-7, 1e-9):
+        s0 = 1.0 - eps
+        dp = np.abs(U.unip_update(x, [m0], [s0], st, 1, "bh2") - at_one_p).max()
+        dc = np.abs(U.unic_update(x, [m0], [s0], mt, st, 1, "bh2") - at_one_c).max()
+        assert dp <= 20 * eps and dc <= 20 * eps, (eps, dp, dc)
+        assert prev_p is None or (dp <= prev_p and dc <= prev_c)
+        prev_p, prev_c = dp, dc
+    # the product's scalar coefficients: same limit, predictor and corrector
+    for corrector in (False, True):
+        one = _Update(st, 1.0, [], corrector, "bh1")
+        near = _Update(st, 1.0 - 1e-9, [], corrector, "bh2")
+        for a, b in ((one.c_x, near.c_x), (one.c_m0, near.c_m0), (one.c_new, near.c_new)):
+            assert abs(a - b) <= 1e-7, (corrector, a, b)
+    u = _Update(st, 1.0, [], True, "bh1")
+    assert abs(u.c_x - st) < 1e-15 and abs(u.c_m0 - 0.5 * (1 - st)) < 1e-15 and abs(u.c_new - 0.5 * (1 - st)) < 1e-15
+
+
 @pytest.mark.parametrize("solver_type", ["bh1", "bh2"])
 def test_solved_updates_are_exact_on_polynomial_data_predictions(solver_type):
     rng = np.random.default_rng(1)

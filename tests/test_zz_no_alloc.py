@@ -30,13 +30,20 @@ def _call_pair(lib, n, H, Hkv, hd, seed, causal_prefix=0):
                                None, causal_prefix, st)
     _lib.check(rc, "cdm_attn_fwd_bf16")
     got = torch.full((n, d), float("nan"), dtype=torch.bfloat16, device=dev())
-    before = torch.cuda.memory_allocated()
-    rc = lib.cdm_attn_fwd_static_bf16(q.data_ptr(), qkv.stride(0), k.data_ptr(), qkv.stride(0), v.data_ptr(),
-                                      qkv.stride(0), cos.data_ptr(), sin.data_ptr(), got.data_ptr(), d, n, H, Hkv, hd,
-                                      None, causal_prefix, st)
-    _lib.check(rc, "cdm_attn_fwd_static_bf16")
+    static = lambda: lib.cdm_attn_fwd_static_bf16(q.data_ptr(), qkv.stride(0), k.data_ptr(), qkv.stride(0), v.data_ptr(),
+                                                  qkv.stride(0), cos.data_ptr(), sin.data_ptr(), got.data_ptr(), d, n, H, Hkv,
+                                                  hd, None, causal_prefix, st)
+    _lib.check(static(), "cdm_attn_fwd_static_bf16")      # the first call on a device resolves the array's address
+    torch.cuda.synchronize()
+    got.fill_(float("nan"))
+    torch.cuda.synchronize()
+    # "allocates nothing" at the level of the device, not only of torch's caching allocator (which a hipMalloc inside the
+    # library would bypass): the free memory the driver reports must not drop across the call
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    _lib.check(static(), "cdm_attn_fwd_static_bf16")
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was allocated inside cdm_attn_fwd_static_bf16"
     return qkv, cos.cpu(), sin.cpu(), got, want
 
 
@@ -56,6 +63,42 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
         kv_end = O.hybrid_kv_end(n, P)[rows] if P else None
         ref = O.attention_rows(qr, kr, x[:, d + dkv:].view(n, Hkv, hd), kv_end).reshape(len(rows), d)
         assert_close(got[rows.to(dev())], ref, BF16_COS, BF16_REL, f"static-scratch attention n={n}")
+
+
+def test_static_scratch_entry_point_under_graph_capture():
+    """The use the entry point is for: recorded into a HIP graph (after cdm_attn_static_scratch_bytes(), which resolves
+    the built-in array on the current device outside the capture), replayed on new inputs - several times, with eager
+    work and synchronisations in between - and compared bit for bit with the eager call on the same inputs."""
+    lib = _lib.load()
+    n, H, Hkv, hd = 900, 4, 2, 128
+    d, dkv = H * hd, Hkv * hd
+    assert lib.cdm_attn_static_scratch_bytes() == 32 << 20
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.zeros((n, d + 2 * dkv), dtype=torch.bfloat16, device=dev())
+    cos, sin = O.mrope_cos_sin(O.text_positions(0, n), hd, (32, 48, 48))
+    cos, sin = cos.contiguous().to(dev()), sin.contiguous().to(dev())
+    out = torch.zeros((n, d), dtype=torch.bfloat16, device=dev())
+    q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
+
+    def call(dst):
+        rc = lib.cdm_attn_fwd_static_bf16(q.data_ptr(), qkv.stride(0), k.data_ptr(), qkv.stride(0), v.data_ptr(), qkv.stride(0),
+                                          cos.data_ptr(), sin.data_ptr(), dst.data_ptr(), d, n, H, Hkv, hd, None, 0,
+                                          torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "cdm_attn_fwd_static_bf16")
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        call(out)
+    for rep in range(3):
+        qkv.copy_((torch.randn(qkv.shape, generator=g) * 0.5).to(torch.bfloat16))
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(out)
+        call(eager)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(out.float()).all())
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
 
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit():
