@@ -106,6 +106,18 @@ __device__ __forceinline__ float tile_row_max(const f32x4 (&s)[KB][QB], int qb) 
     return __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
 }
 
+// Index of the first tile after `after` whose bit is set in the wave's table (bit t of lane l = tile 32 l + t), or a
+// value no tile index reaches.  Wave-uniform.
+__device__ __forceinline__ int next_hot_tile(uint32_t hot, int after, int lane) {
+    const int wl = after >> 5, bit = after & 31;
+    uint32_t w = lane < wl ? 0u : hot;
+    if (lane == wl) w = bit == 31 ? 0u : (w & (~0u << (bit + 1)));
+    const uint64_t lanes = __builtin_amdgcn_ballot_w64(w != 0u);
+    if (lanes == 0) return 0x7fffffff;
+    const int l = __builtin_ctzll(lanes);
+    return 32 * l + __builtin_ctz((uint32_t)__builtin_amdgcn_readlane((int)w, l));
+}
+
 // One pipeline step.  Everything the first MFMAs need is already in registers when the workgroup barrier at
 // the top of the step releases the wave, and all softmax arithmetic is placed under MFMAs:
 //   block A  : S(j+1) = K(j+1) Q^T - m_ref, 32 MFMAs seeded with -m_ref (rolling K fragment window, first
@@ -117,16 +129,18 @@ __device__ __forceinline__ float tile_row_max(const f32x4 (&s)[KB][QB], int qb) 
 //              ||  row maximum of S(j+1) ; first K fragments of tile j+2 (that tile landed before this barrier)
 //   tail     : if some row maximum exceeds the reference by more than 2^kGrowLog2 (rare), move the reference
 //              and rescale O and l.  Scores stay raw (log2 units), so nothing else depends on the reference.
-// The kernel has bounded the scores of its rows (|q| max|k|).  Where no score of the wave's rows can exceed the
-//   reference by more than 2^kSafeLog2, need_max (wave-uniform) is false and the per-tile row maximum and the reference
-//   update are skipped altogether; where the bound fails they run in the tail, after block B (one loop body for both
+// The kernel bounds the scores of its rows against every key tile (|q| max|k| over the tile).  Where no score of the
+//   wave's rows against tile j+1 can exceed the reference by more than 2^kSafeLog2 (wave-uniform, decided per tile
+//   at set-up), the row maximum of that tile and the reference update are skipped; where the bound fails - a
+//   tile with an outlier key, un-normalised huge logits - they run in the tail, after block B (one loop body for both
 //   cases: two copies of the loop do not fit the register budget).
-template <int HD, int QB, class Mid>
-__device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const char* sv_cur, const char* sk_next2,
+template <int HD, int QB, bool LATE, class Mid>
+__device__ __forceinline__ void pipe_step(Mid&& mid, float late_r, const char* sk_next, const char* sv_cur, const char* sk_next2,
                                           const bf16x8 (&qf)[QB][HD / 32], bf16x8 (&kw)[KWIN][KB],
                                           f32x4 (&s_cur)[KB][QB], f32x4 (&s_next)[KB][QB],
                                           f32x4 (&oacc)[HD / 16][QB], f32x4 (&negm)[QB], float (&l_run)[QB], int lane,
-                                          bool next_masked, const int (&next_keys_valid)[QB], bool need_max) {
+                                          bool next_masked, const int (&next_keys_valid)[QB], int next_tile,
+                                          int& next_hot, bool need_always, uint32_t hot) {
     constexpr int KS = HD / 32, HB = HD / 16, NV = 2 * HB;
     // Both blocks are written as a sequence of slots, one MFMA each, fenced so that the compiler keeps them: an odd
     // slot carries one fragment read, an even slot (head_dim 64: every slot) one piece of the softmax arithmetic.
@@ -163,8 +177,9 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
             // the empty asm statements tie the piece to its slot: left alone the compiler gathers all exponentials and
             // conversions of the tile in one place (behind the MFMAs of this block), where nothing overlaps them
             if (e == 0) asm volatile("" : "+v"(s_cur[2 * st + h][q]));
-            const float e0 = __builtin_amdgcn_exp2f(s_cur[2 * st + h][q][e]);
-            const float e1 = __builtin_amdgcn_exp2f(s_cur[2 * st + h][q][e + 1]);
+            // LATE: Q went in scaled by a power of two only (exact), the rest of log2(e)/sqrt(HD) multiplies the fp32 score
+            const float e0 = __builtin_amdgcn_exp2f(LATE ? s_cur[2 * st + h][q][e] * late_r : s_cur[2 * st + h][q][e]);
+            const float e1 = __builtin_amdgcn_exp2f(LATE ? s_cur[2 * st + h][q][e + 1] * late_r : s_cur[2 * st + h][q][e + 1]);
             psum0[q] += e0;
             psum1[q] += e1;
             uint32_t w = pack_bf16x2(e0, e1);
@@ -210,7 +225,10 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
 #pragma unroll
     for (; n_kpre < KWIN * KB; ++n_kpre) kw[n_kpre / KB][n_kpre % KB] = k_frag<HD>(sk_next2, n_kpre / KB, n_kpre % KB, lane);
     __builtin_amdgcn_sched_barrier(0);
-    if (!need_max) return;
+    // tile j + 1 needs row maxima only if it is the wave's next marked tile (one scalar compare on the common path);
+    // the tile after it is looked up behind the maxima (need_always: every tile is the next one)
+    if (next_tile != next_hot) return;
+    next_hot = need_always ? next_tile + 1 : next_hot_tile(hot, next_tile, lane);
     float mx[QB];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) mx[qb] = tile_row_max<QB>(s_next, qb);
@@ -221,7 +239,7 @@ __device__ __forceinline__ void pipe_step(Mid&& mid, const char* sk_next, const 
     for (int qb = 0; qb < QB; ++qb) {
         if (__builtin_amdgcn_ballot_w64(mx[qb] > kGrowLog2) != 0) {
             const float d = mx[qb] > kGrowLog2 ? mx[qb] : 0.0f;
-            const float fac = __builtin_amdgcn_exp2f(-d);
+            const float fac = __builtin_amdgcn_exp2f(LATE ? -d * late_r : -d);      // the probabilities are exp2(late_r s)
             l_run[qb] *= fac;
 #pragma unroll
             for (int hb = 0; hb < HB; ++hb)
@@ -268,7 +286,8 @@ struct PackedParams {
     int n_tokens, n_heads, n_qblocks;
     int kv_group;                // query heads per K / V head (1 = multi-head attention)
     int always_max;              // cross-check: take the row maxima of every tile whatever the norm bound says
-    float scale_log2e;
+    float scale_log2e;           // factor on Q ahead of its rounding to bf16: log2(e)/sqrt(HD), or only its power of two
+    float late_r;                // ... with the rest of it (in [1, 2)) applied to the fp32 scores (LATE kernels)
 };
 
 // QS = query sub-tiles (of 32 rows = two 16-row blocks) per wave: QS = 1 -> 8 waves, two per SIMD, 256 registers each;
@@ -276,7 +295,14 @@ struct PackedParams {
 // four MFMAs instead of two.
 constexpr float kSafeLog2 = 60.0f;      // largest excess over the reference that needs no reference update
 
-template <int HD, int QS>
+// LATE: Q arrives as exact bf16 values that nothing in here touches (no rotation, no norm).  Folding log2(e)/sqrt(HD) into
+// Q would then round every element once more than the reference does (it scales the fp32 scores): percent-level in the
+// probabilities where logits of 50 - 150 compete.  Such calls scale Q by the power-of-two part of the factor (exact)
+// and the fp32 scores by the rest, one multiplication per score; calls that rotate or normalise Q round it once anyway
+// and fold the whole factor into that rounding.
+constexpr int kMaxKm = 2048;            // key tiles that get a decision of their own (131,072 keys); longer sequences: one per head
+
+template <int HD, int QS, bool LATE>
 __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS, 2 / QS))) void attn_fwd_pipe_kernel(
     const PackedParams p) {
     constexpr int NW = 8 / QS;
@@ -290,6 +316,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     constexpr int RING = 3, RING_V = 4;
     __shared__ __attribute__((aligned(1024))) char sk[RING * TILE_BYTES];
     __shared__ __attribute__((aligned(1024))) char sv[RING_V * TILE_BYTES];
+    __shared__ float s_km[kMaxKm];       // largest key norm of every tile of this K / V head, prefix tiles first (set-up only)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -313,16 +340,26 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // ---- Q fragments: rotate-half mRoPE (if tables are given) and the factor log2(e)/sqrt(HD), both in fp32 and
     // with ONE rounding to bf16.  The lane holds channels 32ks + 8g .. +7 (g = lane / 16) of its query row for every
     // ks, so the partner of a channel in k-step ks (< KS/2) is the same register element of k-step ks + KS/2.
-    // An upper bound of every score of a row: |q| max_k |k| (Cauchy-Schwarz on the very bf16 values the
-    // matrix cores multiply).  kmax_all = the largest key norm of this K/V head over all tiles, prefix included.
+    // An upper bound of every score of a row against a key tile: |q| max_{k in tile} |k| (Cauchy-Schwarz on the very
+    // bf16 values the matrix cores multiply).  The per-tile key norms of this K / V head pass through LDS once: each
+    // wave turns them into one bit per tile ("this tile needs row maxima for my rows"), 32 tiles per lane of one
+    // register, and keeps the index of the next such tile in a scalar register: a step compares its tile index with it
+    // (one scalar instruction) and looks the following one up only after a hit.
+    // A sequence of more than kMaxKm tiles falls back to one bound per head (kmax_all).
+    const int NP = p.n_prefix_tiles, NM = (p.n_tokens + BN - 1) / BN;
+    const int NT = NP + NM;
+    const bool per_tile = NT <= kMaxKm;
     float kmax_all = 0.0f;
     {
-        const int nm = (p.n_tokens + BN - 1) / BN;
-        const float* km = p.kmax + (int64_t)kv_head * nm;
-        for (int i = lane; i < nm; i += 64) kmax_all = fmaxf(kmax_all, km[i]);
-        const float* kmp = p.kmax_prefix + (int64_t)kv_head * p.n_prefix_tiles;
-        for (int i = lane; i < p.n_prefix_tiles; i += 64) kmax_all = fmaxf(kmax_all, kmp[i]);
-        kmax_all = wave_max(kmax_all);
+        const float* km = p.kmax + (int64_t)kv_head * NM;
+        const float* kmp = p.kmax_prefix + (int64_t)kv_head * NP;
+        if (per_tile) {
+            for (int i = threadIdx.x; i < kMaxKm; i += 512 / QS) s_km[i] = i >= NT ? 0.0f : (i < NP ? kmp[i] : km[i - NP]);
+        } else {
+            for (int i = lane; i < NM; i += 64) kmax_all = fmaxf(kmax_all, km[i]);
+            for (int i = lane; i < NP; i += 64) kmax_all = fmaxf(kmax_all, kmp[i]);
+            kmax_all = wave_max(kmax_all);
+        }
     }
     float qnorm[QB];
     bf16x8 qf[QB][KS];
@@ -414,8 +451,6 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     }
 
     // key tiles: NP whole tiles of the prefix images, then the NM tiles of the main images
-    const int NP = p.n_prefix_tiles, NM = (p.n_tokens + BN - 1) / BN;
-    const int NT = NP + NM;
     const int n_keys = NP * BN + p.n_tokens;
     const int last_valid = n_keys - (NT - 1) * BN;
     // per-row key limit and the tiles this workgroup needs: a query block inside the causal prefix stops at its
@@ -454,10 +489,12 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     issue(kbase, kpre, sk_addr, 2, 2);
     issue(vbase, vpre, sv_addr, 1, 1);
     issue(vbase, vpre, sv_addr, 2, 2);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(3 * PER_WAVE) : "memory");   // K(0), K(1), V(0) have landed
+    // K(0), K(1), V(0) have landed, and every wave's share of the key-norm table is in LDS
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * PER_WAVE) : "memory");
     f32x4 s_a[KB][QB], s_b[KB][QB];      // score tiles ping-pong between the two halves of the unrolled loop
     const bool ragged = last_valid < BN;
-    bool need_max = p.always_max != 0;
+    bool need_always = p.always_max != 0;
+    float t_lane = INFINITY;      // largest tile key norm this lane's rows tolerate without row maxima
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -467,9 +504,12 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
         const float m0 = tile_row_max<QB>(s_a, qb);      // exact first reference: every row has at least one finite score
-        // can any score of this wave's rows exceed its reference by more than 2^kSafeLog2?  (1 % slack for the fp32
-        // accumulation of the dot products and of the norms; a NaN compares as "yes")
-        need_max = need_max || __builtin_amdgcn_ballot_w64(!(qnorm[qb] * kmax_all * 1.01f - m0 <= kSafeLog2)) != 0;
+        // a tile whose largest key norm is at most thr cannot raise any score of this row more than 2^kSafeLog2 above its
+        // reference (1 % slack for the fp32 accumulation of the dot products and of the norms); a reference that is not
+        // a number asks for the maxima everywhere
+        const float thr = (kSafeLog2 + m0) / (qnorm[qb] * 1.01f);
+        need_always = need_always || __builtin_amdgcn_ballot_w64(thr != thr) != 0;
+        t_lane = fminf(t_lane, thr);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
 #pragma unroll
@@ -477,6 +517,21 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             negm[qb][e] = -m0;
         }
     }
+    float t_wave = t_lane;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) t_wave = fminf(t_wave, __shfl_xor(t_wave, off, 64));
+    if (!per_tile) need_always = need_always || !(kmax_all <= t_wave);
+    uint32_t hot = 0u;      // bit t in lane l: tile 32 l + t needs row maxima for this wave's rows
+    if (per_tile && !need_always) {
+#pragma unroll
+        for (int c4 = 0; c4 < 8; ++c4) {
+            const float4 v = *reinterpret_cast<const float4*>(&s_km[32 * lane + 4 * c4]);
+            hot |= (uint32_t)(!(v.x <= t_wave)) << (4 * c4) | (uint32_t)(!(v.y <= t_wave)) << (4 * c4 + 1) |
+                   (uint32_t)(!(v.z <= t_wave)) << (4 * c4 + 2) | (uint32_t)(!(v.w <= t_wave)) << (4 * c4 + 3);
+        }
+    }
+    // tile 0 had its exact maxima above; need_always = every tile is "the next one"
+    int next_hot = need_always ? 1 : next_hot_tile(hot, 0, lane);
     bf16x8 kw[KWIN][KB];
     preload_k<HD>(sk + TILE_BYTES, kw, lane);      // K(1) for step 0
 
@@ -509,10 +564,11 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QB];                                                                                         \
         _Pragma("unroll") for (int qb = 0; qb < QB; ++qb) nvalid[qb] = klim[qb] - (j + 1) * BN;                 \
-        pipe_step<HD, QB>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); },               \
+        /* does tile j + 1 (the scores block A computes) need row maxima?  its bit of the wave's table */      \
+        pipe_step<HD, QB, LATE>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); }, p.late_r,       \
                           sk + ks_next * TILE_BYTES, sv + v_cur * TILE_BYTES, sk + k_next2 * TILE_BYTES, qf, kw, \
                           SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 >= NT), nvalid,   \
-                          need_max);                                                                            \
+                          j + 1, next_hot, need_always, hot);     /* tile j + 1: the scores block A computes */ \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         if (late_sync) load_v();                                                                                \
         ks_cur = ks_next;                                                                                       \
@@ -785,7 +841,13 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     p.cos = cos; p.sin = sin;
     p.qn = qn;
     p.n_tokens = (int)n_tokens; p.n_heads = n_heads; p.kv_group = n_heads / n_kv_heads;
-    p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
+    // Q untouched by rotation and norm: only the power-of-two part of the factor goes into Q (see LATE above)
+    const bool late = cos == nullptr && qk_norm == nullptr;
+    const float full = 1.4426950408889634f / sqrtf((float)head_dim);
+    int ex = 0;
+    const float mant = frexpf(full, &ex);                 // full = mant * 2^ex, mant in [0.5, 1)
+    p.scale_log2e = late ? ldexpf(1.0f, ex - 1) : full;
+    p.late_r = late ? 2.0f * mant : 1.0f;
     p.n_qblocks = (int)((n_tokens + BMQ - 1) / BMQ);
     // 1-D grid of 8 x ceil(heads / 8) x query blocks ids: id % 8 = XCD, see the kernel's placement rule
     const int64_t nwg = 8ll * ((n_heads + 7) / 8) * p.n_qblocks;
@@ -796,9 +858,11 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     // cross-check build only: 1 = 64 query rows per wave (4 waves), 2 = variant 0 with the row maxima always taken
     const int variant = cdm_get_variant(0);
     p.always_max = variant == 2;
-#define CDM_ATTN_LAUNCH(QS_, THREADS)                                                   \
-    if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_><<<grid, THREADS, 0, st>>>(p);  \
-    else attn_fwd_pipe_kernel<64, QS_><<<grid, THREADS, 0, st>>>(p)
+#define CDM_ATTN_LAUNCH(QS_, THREADS)                                                                      \
+    if (head_dim == 128 && late) attn_fwd_pipe_kernel<128, QS_, true><<<grid, THREADS, 0, st>>>(p);       \
+    else if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_, false><<<grid, THREADS, 0, st>>>(p);         \
+    else if (late) attn_fwd_pipe_kernel<64, QS_, true><<<grid, THREADS, 0, st>>>(p);                      \
+    else attn_fwd_pipe_kernel<64, QS_, false><<<grid, THREADS, 0, st>>>(p)
 #ifdef CDM_CROSSCHECK
     if (variant == 1) { CDM_ATTN_LAUNCH(2, 256); }
     else

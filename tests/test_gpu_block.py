@@ -248,6 +248,59 @@ def test_c1_full_size_attention_sampled_rows():
         assert torch.equal(o, again), "attention output differs between identical launches"
 
 
+def test_full_size_attention_with_outlier_keys():
+    """56,832 tokens (the joint length of benchmark configuration 2), 32 heads x 128, mRoPE in registers, with one
+    outlier key in each of two heads.  The kernel decides per key tile and per wave whether the tile's key-norm bound
+    allows it to skip the row maxima: head 0 gets an outlier whose norm is the MEDIAN of the waves' thresholds, so in
+    that one tile about half of the waves of every workgroup take the maxima and the others do not (mixed waves in
+    one workgroup, at full size); head 13 gets a key of norm 4000 that beats everything else by far more than 2^60
+    for many rows (the reference moves by a hundred and more).  All other tiles of both heads, and every tile of the other
+    heads, run without maxima.  Sampled rows against the fp32 oracle, and bit-reproducibility."""
+    cfg = CONFIGS["C2"]
+    n, H, hd, d = cfg.n_tokens, cfg.n_heads, cfg.head_dim, cfg.d_model
+    g = torch.Generator(device=dev()).manual_seed(77)
+    qkv = (torch.randn((n, 3 * d), generator=g, device=dev()) / (hd ** 0.5)).to(torch.bfloat16)
+    pos, _ = rotary.build_positions(cfg.n_text, cfg.grid)
+    cos, sin = rotary.rotary_tables(pos, hd, cfg.mrope_sections)
+    cg, sg = cos.to(dev()), sin.to(dev())
+    # the waves' thresholds in head 0, restated on the host: a wave owns 32 consecutive query rows; a row tolerates a
+    # tile whose largest key norm is at most (60 + m0) / (1.01 |q'|), q' = rotated Q times log2(e)/sqrt(hd), m0 = its
+    # largest score against the first 64 keys
+    c = 1.4426950408889634 / hd ** 0.5
+    q0 = O.apply_mrope(qkv[:, :hd].float().view(n, 1, hd), cg, sg).view(n, hd) * c
+    k0 = O.apply_mrope(qkv[:64, d:d + hd].float().view(64, 1, hd), cg[:64], sg[:64]).view(64, hd)
+    thr = (60.0 + (q0 @ k0.t()).amax(1)) / (1.01 * q0.norm(dim=1))
+    t_wave = thr.view(-1, 32).amin(1)
+    spike0 = float(t_wave.median())
+    assert 100.0 < spike0 < 2000.0
+    per_wg = (t_wave.view(-1, 8) >= spike0).float().mean(1)
+    assert float(((per_wg > 0) & (per_wg < 1)).float().mean()) > 0.9      # both kinds of waves in most workgroups
+    at0, at13 = 40000, 100
+    u = torch.randn(2, hd, generator=g, device=dev())
+    u = u / u.norm(dim=1, keepdim=True)
+    qkv[at0, d:d + hd] = (u[0] * spike0).to(torch.bfloat16)
+    qkv[at13, d + 13 * hd:d + 14 * hd] = (u[1] * 4000.0).to(torch.bfloat16)
+    q, k, v = qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:]
+    o = ops.attention(q, k, v, H, hd, cos=cg, sin=sg)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(o.float()).all())
+    rows = torch.cat([torch.tensor([0, 1, 31, 32, 255, 256, n - 1, n - 64, at0, at13]),
+                      torch.randint(0, n, (54,), generator=torch.Generator().manual_seed(2))])
+    for h in (0, 13, 5):
+        sl = slice(h * hd, (h + 1) * hd)
+        kr = O.apply_mrope(qkv[:, d + h * hd:d + (h + 1) * hd].float().cpu().view(n, 1, hd), cos, sin)
+        qr = O.apply_mrope(qkv[rows.to(dev()), sl].float().cpu().view(-1, 1, hd), cos[rows], sin[rows])
+        vr = qkv[:, 2 * d + h * hd:2 * d + (h + 1) * hd].float().cpu().view(n, 1, hd)
+        want = O.attention_rows(qr, kr, vr).reshape(-1, hd)
+        if h == 13:      # the spike decides many rows: they return (nearly) V of the outlier key
+            sc = (qr.view(-1, hd) @ kr.view(n, hd).t()) * c
+            assert int(((sc[:, at13] - sc.amax(1)) == 0).sum()) >= 10 and float(sc[:, at13].amax()) > 80.0
+        assert_close(o[rows.to(dev()), sl], want, BF16_COS, BF16_REL, f"full-size attention with outlier keys, head {h}")
+    for _ in range(3):
+        again = ops.attention(q, k, v, H, hd, cos=cg, sin=sg)
+        assert torch.equal(o, again), "attention output differs between identical launches"
+
+
 def test_transformer_with_stack_edges_and_loaded_checkpoint(tmp_path):
     """latents -> patchify/proj_in -> 2 MoT blocks (QK-norm) -> final norm -> proj_out/unpatchify, with the weights
     taken through a safetensors file; checked against the fp32 oracle composed from the same tensors."""
