@@ -466,8 +466,10 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     const int kmax = (causal_wg && b0 + BMQ <= p.causal_prefix) ? (b0 + BMQ < n_keys ? b0 + BMQ : n_keys) : n_keys;
     const int NTW = (kmax + BN - 1) / BN;
     const uint32_t lane_off = (uint32_t)(wave * 1024 + lane * 16);
-    const char* kbase = p.kp + (int64_t)kv_head * NM * TILE_BYTES;
-    const char* vbase = p.vp + (int64_t)kv_head * NM * TILE_BYTES;
+    // tile t of the key sequence [prefix tiles | main tiles] lives at pre + t * TILE_BYTES (t < NP) or at
+    // base + t * TILE_BYTES with base shifted back by the prefix length: one 32-bit offset serves both
+    const char* kbase = p.kp + ((int64_t)kv_head * NM - NP) * TILE_BYTES;
+    const char* vbase = p.vp + ((int64_t)kv_head * NM - NP) * TILE_BYTES;
     const char* kpre = p.kp_prefix + (int64_t)kv_head * NP * TILE_BYTES;
     const char* vpre = p.vp_prefix + (int64_t)kv_head * NP * TILE_BYTES;
     const uint32_t sk_addr = lds_addr_of(sk) + wave * 1024, sv_addr = lds_addr_of(sv) + wave * 1024;
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // vmcnt arithmetic below stays valid at the end of the sequence) -> ring slot `slot`
     auto issue = [&](const char* base, const char* pre, uint32_t dst_addr, int t, int slot) {
         const int tc = t < NT ? t : NT - 1;
-        const char* src = tc < NP ? pre + (int64_t)tc * TILE_BYTES : base + (int64_t)(tc - NP) * TILE_BYTES;
+        const char* src = (tc < NP ? pre : base) + (uint32_t)tc * (uint32_t)TILE_BYTES;      // images stay below 4 GB per head
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i)
             lds_dma16(src + i * (NW * 1024), lane_off, dst_addr + slot * TILE_BYTES + i * (NW * 1024));
