@@ -44,10 +44,11 @@ SIGNATURES = {
     "cdm_adaln_rmsnorm_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
     "cdm_adaln_rmsnorm_f32_quant_e4m3": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I64, _F32, _P]),
     "cdm_quant_rows_e4m3": (_I32, [_P, _I64, _P, _P, _I64, _I64, _P]),
+    "cdm_quant_rows_from_parts_e4m3": (_I32, [_P, _I64, _P, _I64, _I64, _P, _P, _I64, _I64, _P]),
     "cdm_gemm_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P, _P, _P, _I64,
                              _I32, _P]),
     "cdm_gemm_fp8": (_I32, [_P, _I64, _P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I32, _P, _I64, _P, _P,
-                            _P, _I64, _I32, _P]),
+                            _P, _I64, _I32, _P, _I64, _P]),
     "cdm_mrope_qk_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I32, _I32, _P]),
     "cdm_attn_workspace_bytes": (_I64, [_I64, _I32, _I32]),
     "cdm_attn_fwd_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _I64, _P, _I64,
@@ -55,10 +56,10 @@ SIGNATURES = {
     "cdm_attn_static_scratch_bytes": (_I64, []),
     "cdm_attn_fwd_static_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _I64, _P]),
     "cdm_attn_pack_kv_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _P]),
-    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _P, _I64, _I64, _P]),
+    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _P, _I64, _I64, _P, _P]),
     "cdm_grouped_gemm_fp8": (_I32, [_P, _I64, _P, C.POINTER(_P), C.POINTER(_P), _I64, C.POINTER(_P), C.POINTER(_P), _P, _I64,
                                     C.POINTER(_I64), C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P,
-                                    _P, _I64, _I32, _P]),
+                                    _P, _I64, _I32, _P, _I64, _P]),
     "cdm_cfg_step_f32": (_I32, [_P, _P, _P, _F32, C.POINTER(_P), _I32, C.POINTER(_F32), C.POINTER(_P), _I32, _I64, _P]),
     "cdm_grouped_gemm_qkv_pack_bf16": (_I32, [_P, _I64, C.POINTER(_P), _I64, _P, _I64, C.POINTER(_I64), C.POINTER(_I64), _I32,
                                               _I64, _I32, _I32, _I32, _P, _P, _P, _P, _I64, _P]),

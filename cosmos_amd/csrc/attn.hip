@@ -281,6 +281,7 @@ struct PackedParams {
     int n_prefix_tiles;
     int causal_prefix;           // query rows < causal_prefix see keys <= their own index only; the others see all keys
     bf16_t* o; int64_t ldo;
+    float* row_amax;             // optional [n_tokens, n_heads]: largest |o| of each output row within each head (as stored)
     const float* cos; const float* sin;   // optional rotary tables [n_tokens, HD/2] applied to Q at load
     QkNormDev qn;                          // optional per-head RMSNorm of Q, applied before the rotation
     int n_tokens, n_heads, n_qblocks;
@@ -594,12 +595,20 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
         l_tot += __shfl_xor(l_tot, 32, 64);
         const float inv = 1.0f / l_tot;
+        float amax = 0.0f;
 #pragma unroll
         for (int hb = 0; hb < HB; ++hb) {
             uint2 w;
             w.x = pack_bf16x2(oacc[hb][qb][0] * inv, oacc[hb][qb][1] * inv);
             w.y = pack_bf16x2(oacc[hb][qb][2] * inv, oacc[hb][qb][3] * inv);
             *reinterpret_cast<uint2*>(stage + (qb * 16 + r16) * PITCH + (16 * hb + 4 * g4) * 2) = w;
+            amax = fmaxf(fmaxf(amax, fmaxf(fabsf(bf16lo(w.x)), fabsf(bf16hi(w.x)))), fmaxf(fabsf(bf16lo(w.y)), fabsf(bf16hi(w.y))));
+        }
+        if (p.row_amax != nullptr) {      // the row's channels of this head are spread over the four quarter-waves
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            const int qrow = q0 + qb * 16 + r16;
+            if (g4 == 0 && qrow < p.n_tokens) p.row_amax[(int64_t)qrow * p.n_heads + head] = amax;
         }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
@@ -807,8 +816,10 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
                                             const void* workspace, void* o, int64_t ldo, int64_t n_tokens,
                                             int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
                                             const cdm_qk_norm* qk_norm, const void* prefix_workspace,
-                                            int64_t n_prefix_tokens, int64_t causal_prefix, void* stream) {
+                                            int64_t n_prefix_tokens, int64_t causal_prefix, float* row_amax,
+                                            void* stream) {
     CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
+    CDM_REQUIRE((reinterpret_cast<uintptr_t>(row_amax) & 3u) == 0, CDM_ERR_BAD_ALIGN, "attn_fwd_packed: row_amax must be 4-byte aligned");
     CDM_REQUIRE(n_kv_heads > 0 && n_heads > 0 && n_heads % n_kv_heads == 0, CDM_ERR_BAD_SHAPE,
                 "attn_fwd_packed: n_kv_heads=%d must divide n_heads=%d", n_kv_heads, n_heads);
     CDM_REQUIRE(n_prefix_tokens >= 0 && n_prefix_tokens % BN == 0 && n_prefix_tokens < (1ll << 23), CDM_ERR_BAD_SHAPE,
@@ -840,6 +851,7 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     p.n_prefix_tiles = (int)(n_prefix_tokens / BN);
     p.causal_prefix = (int)causal_prefix;
     p.o = (bf16_t*)o; p.ldo = ldo;
+    p.row_amax = row_amax;
     p.cos = cos; p.sin = sin;
     p.qn = qn;
     p.n_tokens = (int)n_tokens; p.n_heads = n_heads; p.kv_group = n_heads / n_kv_heads;
@@ -905,7 +917,7 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
                                     qk_norm, stream)))
         return rc;
     return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, n_kv_heads, head_dim, qk_norm,
-                                    nullptr, 0, causal_prefix, stream);
+                                    nullptr, 0, causal_prefix, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -58,6 +58,9 @@ struct GemmParams {
     char* kp; char* vp; float* kmax;
     int d_q, d_kv, n_key_tiles;
     float k_eps;                         // epsilon of the per-head RMSNorm of K (segments with a weight row)
+    // CDM_EPI_SWIGLU, optional: [M, amax_ld] fp32, entry (row, c) = largest |output| of the row within output columns
+    // 64 c .. 64 c + 63 (as stored): what a per-row quantiser of the output needs, without a pass of its own
+    float* row_amax; int64_t amax_ld;
     int tiles_n, total_tiles, n_seg;
     GemmSeg seg[kMaxSeg];
 };
@@ -259,6 +262,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
             if (row >= t.m_end) continue;
             const float sr = FP8 ? p.sa[row] : 1.0f;
             bf16_t* crow = p.C + (int64_t)row * p.ldc;
+            float amax = 0.0f;
 #pragma unroll
             for (int cs = 0; cs < HALF; ++cs) {
                 const int cl = ACC::col_local(cs, lane), col = colw + cl;
@@ -276,6 +280,12 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
                 const uint2 o2 = pack4_bf16(o[0], o[1], o[2], o[3]);
                 if (stage) *reinterpret_cast<uint2*>(stage + rl * kStagePitch + cl * 2) = o2;
                 else *reinterpret_cast<uint2*>(crow + col) = o2;
+                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(bf16lo(o2.x)), fabsf(bf16hi(o2.x)))), fmaxf(fabsf(bf16lo(o2.y)), fabsf(bf16hi(o2.y))));
+            }
+            if (p.row_amax != nullptr) {      // lanes r, r + 16, r + 32, r + 48 hold the row's 64 columns of this piece
+                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                if ((lane >> 4) == 0 && colw < p.N) p.row_amax[(int64_t)row * p.amax_ld + (colw >> 6)] = amax;
             }
         }
         if (stage) copy_out<64, 2, ROWS>(p, t, stage, row0, colw, lane);
@@ -848,13 +858,18 @@ int32_t grouped(const char* who, const void* A, int64_t lda, const float* sa, co
                 const int64_t* seg_start, const int64_t* seg_len, int32_t n_seg, int64_t N, int64_t K, int32_t epilogue,
                 const void* R, int64_t ldr, const float* const* gate, const float* cos, const float* sin,
                 int64_t rope_cols, int32_t head_dim, void* stream, const GemmParams* pack = nullptr,
-                const float* k_norm_rows = nullptr) {
+                const float* k_norm_rows = nullptr, float* row_amax = nullptr, int64_t amax_ld = 0) {
     constexpr int esize = FP8 ? 1 : 2;
     CDM_REQUIRE(A && W && C && seg_start && seg_len, CDM_ERR_BAD_ARG, "%s: null pointer", who);
     CDM_REQUIRE((epilogue == CDM_EPI_QKV_PACK) == (pack != nullptr), CDM_ERR_BAD_ARG,
                 "%s: the QKV_PACK epilogue belongs to the qkv_pack entry points", who);
     CDM_REQUIRE(n_seg >= 0 && n_seg <= 64, CDM_ERR_BAD_ARG, "%s: n_seg=%d out of range", who, n_seg);
     if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(W2, CDM_ERR_BAD_ARG, "%s: SWIGLU needs W2", who);
+    if (row_amax != nullptr) {
+        CDM_REQUIRE(epilogue == CDM_EPI_SWIGLU, CDM_ERR_BAD_ARG, "%s: row_amax belongs to the SWIGLU epilogue", who);
+        CDM_REQUIRE((reinterpret_cast<uintptr_t>(row_amax) & 3u) == 0 && amax_ld >= (N + 63) / 64, CDM_ERR_BAD_ARG,
+                    "%s: row_amax must be 4-byte aligned with a row stride of at least ceil(N / 64)", who);
+    }
     if (FP8) {
         CDM_REQUIRE(sa && sw, CDM_ERR_BAD_ARG, "%s: null scale pointer", who);
         if (epilogue == CDM_EPI_SWIGLU) CDM_REQUIRE(sw2, CDM_ERR_BAD_ARG, "%s: SWIGLU needs sw2", who);
@@ -890,6 +905,7 @@ int32_t grouped(const char* who, const void* A, int64_t lda, const float* sa, co
     p.N = (int)N; p.K = (int)K;
     p.R = (const bf16_t*)R; p.ldr = ldr;
     p.cos = cos; p.sin = sin; p.rope_cols = (int)rope_cols; p.head_dim = head_dim;
+    p.row_amax = row_amax; p.amax_ld = amax_ld;
     if (pack) {
         p.kp = pack->kp; p.vp = pack->vp; p.kmax = pack->kmax;
         p.d_q = pack->d_q; p.d_kv = pack->d_kv; p.n_key_tiles = pack->n_key_tiles; p.k_eps = pack->k_eps;
@@ -984,13 +1000,13 @@ extern "C" int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, co
                                 const float* sw, const void* W2q, const float* sw2, void* C, int64_t ldc, int64_t M,
                                 int64_t N, int64_t K, int32_t epilogue, const void* R, int64_t ldr, const float* gate,
                                 const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
-                                void* stream) {
+                                float* row_amax, int64_t amax_ld, void* stream) {
     const int64_t start = 0;
     const void* w2[1] = {W2q};
     const float* s2[1] = {sw2};
     CDM_REQUIRE(sa && sw, CDM_ERR_BAD_ARG, "gemm_fp8: null scale pointer");
     return grouped<true>("gemm_fp8", Aq, lda, sa, &Wq, &sw, ldw, W2q ? w2 : nullptr, s2, C, ldc, &start, &M, 1, N, K, epilogue,
-                         R, ldr, &gate, cos, sin, rope_cols, head_dim, stream);
+                         R, ldr, &gate, cos, sin, rope_cols, head_dim, stream, nullptr, nullptr, row_amax, amax_ld);
 }
 
 extern "C" int32_t cdm_grouped_gemm_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw,
@@ -1008,7 +1024,8 @@ extern "C" int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float
                                         const float* const* sw2, void* C, int64_t ldc, const int64_t* seg_start,
                                         const int64_t* seg_len, int32_t n_seg, int64_t N, int64_t K, int32_t epilogue,
                                         const void* R, int64_t ldr, const float* const* gate, const float* cos,
-                                        const float* sin, int64_t rope_cols, int32_t head_dim, void* stream) {
+                                        const float* sin, int64_t rope_cols, int32_t head_dim, float* row_amax,
+                                        int64_t amax_ld, void* stream) {
     return grouped<true>("grouped_gemm_fp8", Aq, lda, sa, Wq, sw, ldw, W2q, sw2, C, ldc, seg_start, seg_len, n_seg, N, K,
-                         epilogue, R, ldr, gate, cos, sin, rope_cols, head_dim, stream);
+                         epilogue, R, ldr, gate, cos, sin, rope_cols, head_dim, stream, nullptr, nullptr, row_amax, amax_ld);
 }

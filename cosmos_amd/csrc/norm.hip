@@ -189,6 +189,53 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(const bf16_t* __re
     }
 }
 
+// the same quantisation where the producer of `a` left partial row maxima behind ([rows, n_parts], entry = largest |a|
+// of the row within one column range): the row is read once
+__global__ __launch_bounds__(kThreads) void quant_rows_parts_kernel(const bf16_t* __restrict__ a, int64_t lda,
+                                                                    const float* __restrict__ parts, int64_t ldp, int n_parts,
+                                                                    uint8_t* __restrict__ q, float* __restrict__ s,
+                                                                    int64_t rows, int cols) {
+    __shared__ float slot_max[2][4];
+    int par = 0;
+    const int nchunk = cols >> 3;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const uint4* ar = reinterpret_cast<const uint4*>(a + row * lda);
+        // the row's first chunks are requested before the maxima are reduced (eight per thread in flight: 32 KB of a row)
+        constexpr int PRE = 8;
+        uint4 raw[PRE];
+#pragma unroll
+        for (int c = 0; c < PRE; ++c) {
+            const int idx = c * kThreads + threadIdx.x;
+            raw[c] = idx < nchunk ? ar[idx] : make_uint4(0, 0, 0, 0);
+        }
+        float amax = 0.0f;
+        for (int i = threadIdx.x; i < n_parts; i += kThreads) amax = fmaxf(amax, parts[row * ldp + i]);
+        amax = block_reduce<true>(amax, slot_max, par);
+        float sc = amax / kE4M3Max;
+        if (sc == 0.0f) sc = 1.0f;
+        if (threadIdx.x == 0) s[row] = sc;
+        uint2* qr = reinterpret_cast<uint2*>(q + row * (int64_t)cols);
+#pragma unroll
+        for (int c = 0; c < PRE; ++c) {
+            const int idx = c * kThreads + threadIdx.x;
+            if (idx < nchunk) {
+                float f[8];
+                unpack8(raw[c], f);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = f[i] / sc;
+                qr[idx] = pack_e4m3x8(f);
+            }
+        }
+        for (int idx = PRE * kThreads + threadIdx.x; idx < nchunk; idx += kThreads) {
+            float f[8];
+            unpack8(ar[idx], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = f[i] / sc;
+            qr[idx] = pack_e4m3x8(f);
+        }
+    }
+}
+
 template <bool QUANT, bool XF32>
 int32_t launch_norm(const void* x, const void* w, const float* shift, const float* scale, void* y, float* s_tok,
                     int64_t n_tokens, int64_t d, float eps, hipStream_t st) {
@@ -273,4 +320,25 @@ extern "C" int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, floa
     quant_rows_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>((const bf16_t*)a, lda, (uint8_t*)q, s, rows,
                                                                   (int)cols);
     return cdm_check_launch("quant_rows");
+}
+
+extern "C" int32_t cdm_quant_rows_from_parts_e4m3(const void* a, int64_t lda, const float* parts, int64_t ldp,
+                                                  int64_t n_parts, void* q, float* s, int64_t rows, int64_t cols,
+                                                  void* stream) {
+    CDM_REQUIRE(a && q && s && parts, CDM_ERR_BAD_ARG, "quant_rows_from_parts: null pointer");
+    CDM_REQUIRE(rows >= 0 && cols > 0 && lda >= cols, CDM_ERR_BAD_ARG, "quant_rows_from_parts: bad sizes");
+    CDM_REQUIRE(n_parts >= 1 && n_parts <= 4096 && ldp >= n_parts, CDM_ERR_BAD_ARG,
+                "quant_rows_from_parts: n_parts=%lld must be 1..4096 with ldp >= n_parts", (long long)n_parts);
+    CDM_REQUIRE(cols % 8 == 0 && cols <= 32768, CDM_ERR_BAD_SHAPE,
+                "quant_rows_from_parts: cols=%lld must be a multiple of 8 and <= 32768", (long long)cols);
+    CDM_REQUIRE(cdm_aligned16(a) && cdm_aligned16(q) && (lda % 8 == 0) && (reinterpret_cast<uintptr_t>(parts) & 3u) == 0,
+                CDM_ERR_BAD_ALIGN, "quant_rows_from_parts: pointers/strides must be 16-byte aligned (parts: 4-byte)");
+    int32_t rc = cdm_require_device();
+    if (rc) return rc;
+    if (rows == 0) return CDM_OK;
+    const int64_t max_blocks = 256 * 8;
+    const int grid = (int)(rows < max_blocks ? rows : max_blocks);
+    quant_rows_parts_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>((const bf16_t*)a, lda, parts, ldp, (int)n_parts,
+                                                                        (uint8_t*)q, s, rows, (int)cols);
+    return cdm_check_launch("quant_rows_from_parts");
 }

@@ -72,6 +72,10 @@ class Workspace:
             self.yq, self.ys = torch.empty((n, d), **q8), torch.empty((n,), **f32)
             self.oq, self.os = torch.empty((n, d), **q8), torch.empty((n,), **f32)
             self.hq, self.hs = torch.empty((n, hidden), **q8), torch.empty((n,), **f32)
+            # partial row maxima the producing kernels leave for the quantisers: per head (attention output) and per 64
+            # columns (SwiGLU hidden)
+            self.o_amax = torch.empty((n, n_heads), **f32)
+            self.h_amax = torch.empty((n, (hidden + 63) // 64), **f32)
         self.y = torch.empty((n, d), **bf)
         self.qkv = torch.empty((n, d + 2 * n_kv_heads * head_dim), **bf)       # [Q | K | V] columns
         self.attn_out = torch.empty((n, d), **bf)
@@ -145,6 +149,7 @@ class DMAttnProcessor:
         mask_kw = dict(causal_prefix=causal_prefix, prefix=prefix, n_kv_heads=attn.n_kv_heads)
         q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
         qkn = attn.qk_norm_args(modality_segments)
+        o_amax = None      # per-head maxima of the attention output rows, where the attention kernel leaves them
         if qkn is not None and self.rope != "in_attention":
             raise NotImplementedError("QK-RMSNorm precedes the rotation: it needs rope='in_attention'")
         if self.rope == "gemm_epilogue":
@@ -157,8 +162,9 @@ class DMAttnProcessor:
                 wsb = torch.empty((ops.attn_workspace_bytes(n, attn.n_kv_heads, attn.head_dim),), dtype=torch.uint8,
                                   device=x.device)
             attn._qkv_pack(x, quant_scale, modality_segments, qkv, wsb, cos, sin, qkn)
+            o_amax = ws.o_amax if (attn.fp8 and ws is not None and ws.fp8) else None
             ops.attention_packed(q, wsb, attn.n_heads, attn.head_dim, o, cos, sin, qkn, prefix, causal_prefix,
-                                 attn.n_kv_heads)
+                                 attn.n_kv_heads, row_amax=o_amax)
         else:
             attn._linear(x, quant_scale, "qkv", modality_segments, out=qkv, epilogue="none")
             if self.rope == "streaming":
@@ -171,7 +177,9 @@ class DMAttnProcessor:
             else:     # in registers, inside the attention kernels
                 ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, cos=cos, sin=sin,
                               qk_norm=qkn, **mask_kw)
-        if attn.fp8:
+        if attn.fp8 and o_amax is not None:
+            oq, so = ops.quant_rows_from_parts(o, o_amax, ws.oq, ws.os)
+        elif attn.fp8:
             oq, so = ops.quant_rows(o, ws.oq, ws.os) if ws is not None and ws.fp8 else ops.quant_rows(o)
         else:
             oq, so = o, None
@@ -367,7 +375,7 @@ class DMAttention(nn.Module, _AttentionCore):
 
 
 def _routed_linear(a, sa, weights, qweights, weights2, segments, *, out, epilogue, residual=None, gates=None, cos=None,
-                   sin=None, rope_cols=0, head_dim=0, qweights2=None) -> None:
+                   sin=None, rope_cols=0, head_dim=0, qweights2=None, row_amax=None) -> None:
     """Per-modality linear over contiguous token segments: one grouped launch over all segments."""
     segl = [(s, l) for (s, l, _, _) in segments]
     if qweights is None:
@@ -388,7 +396,7 @@ def _routed_linear(a, sa, weights, qweights, weights2, segments, *, out, epilogu
                          segl, w2qs=[qweights2[b][0] for (_, _, b, _) in segments] if qweights2 is not None else None,
                          sw2s=[qweights2[b][1] for (_, _, b, _) in segments] if qweights2 is not None else None,
                          epilogue=epilogue, residual=residual, gates=gates, cos=cos, sin=sin, rope_cols=rope_cols,
-                         head_dim=head_dim, out=out)
+                         head_dim=head_dim, out=out, row_amax=row_amax)
 
 
 class DMBlock(nn.Module):
@@ -477,9 +485,9 @@ class DMBlock(nn.Module):
         y, sy = self._norm(x, self.norm2_weight, sh2, sc2, segs, ws)
         q = self._q if self.fp8 else {}
         _routed_linear(y, sy, self.gate_weight, q.get("gate"), self.up_weight, segs, out=ws.h, epilogue="swiglu",
-                       qweights2=q.get("up"))
-        if self.fp8:
-            hq, sh = ops.quant_rows(ws.h, ws.hq, ws.hs)
+                       qweights2=q.get("up"), row_amax=ws.h_amax if self.fp8 else None)
+        if self.fp8:      # the SwiGLU epilogue left the maxima of every 64 columns: the quantiser reads each row once
+            hq, sh = ops.quant_rows_from_parts(ws.h, ws.h_amax, ws.hq, ws.hs)
         else:
             hq, sh = ws.h, None
         gates = [g2 if modulated else None for (_, _, _, modulated) in segs]

@@ -151,6 +151,37 @@ def quant_rows(a: torch.Tensor, out_q: Optional[torch.Tensor] = None,
     return q, s
 
 
+@_timed("quant")
+def quant_rows_from_parts(a: torch.Tensor, parts: torch.Tensor, out_q: Optional[torch.Tensor] = None,
+                          out_s: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``quant_rows`` (same result, bit for bit) from partial row maxima the producer of ``a`` left behind: ``parts``
+    [rows, n_parts] fp32, entry (i, c) = max |a[i, j]| over one column range, the ranges covering the row
+    (``attention_packed(row_amax=...)``: one per head; ``gemm_fp8(epilogue="swiglu", row_amax=...)``: one per 64
+    columns).  The row is read once."""
+    lib = _lib.load()
+    rows, cols = a.shape
+    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=a.device) if out_q is None else out_q
+    s = torch.empty((rows,), dtype=torch.float32, device=a.device) if out_s is None else out_s
+    if q.shape != (rows, cols) or not q.is_contiguous() or s.shape != (rows,) or not s.is_contiguous():
+        raise ValueError("out_q / out_s must be contiguous [rows, cols] e4m3 and [rows] fp32")
+    if parts.dim() != 2 or parts.shape[0] != rows:
+        raise ValueError("parts must be [rows, n_parts]")
+    rc = lib.cdm_quant_rows_from_parts_e4m3(_chk(a, "a", torch.bfloat16, 2), a.stride(0), _chk(parts, "parts", torch.float32, 2),
+                                            parts.stride(0), parts.shape[1], _chk(q, "out_q", FP8_DTYPE, 2),
+                                            _chk(s, "out_s", torch.float32, 1), rows, cols, _stream())
+    _lib.check(rc, "cdm_quant_rows_from_parts_e4m3")
+    return q, s
+
+
+def _amax_arg(row_amax: Optional[torch.Tensor], rows: int, min_cols: int):
+    """(pointer, row stride) of an optional [rows, >= min_cols] fp32 output of partial row maxima."""
+    if row_amax is None:
+        return None, 0
+    if row_amax.dim() != 2 or row_amax.shape[0] != rows or row_amax.shape[1] < min_cols:
+        raise ValueError(f"row_amax must be [{rows}, >= {min_cols}] fp32")
+    return _chk(row_amax, "row_amax", torch.float32, 2), row_amax.stride(0)
+
+
 # ----------------------------------------------------------------------------- GEMM
 @_timed("gemm")
 def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, epilogue: str = "none",
@@ -185,8 +216,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
 def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, *,
              w2q: Optional[torch.Tensor] = None, sw2: Optional[torch.Tensor] = None, epilogue: str = "none",
              residual=None, gate=None, cos=None, sin=None, rope_cols: int = 0, head_dim: int = 0,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[M, N] = epilogue((aq @ wq^T) * sa[:, None] * sw[None, :]); e4m3 operands, bf16 out."""
+             out: Optional[torch.Tensor] = None, row_amax: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = epilogue((aq @ wq^T) * sa[:, None] * sw[None, :]); e4m3 operands, bf16 out.  ``row_amax`` (SwiGLU
+    epilogue only): [M, >= ceil(N / 64)] fp32 that receives the largest |out| of each row within every 64 columns."""
     lib = _lib.load()
     M, K = aq.shape
     N = wq.shape[0]
@@ -201,7 +233,7 @@ def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Ten
                           _chk(residual, "residual", odt, 2),
                           residual.stride(0) if residual is not None else 0, _f32vec(gate, "gate", N),
                           _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols), int(head_dim),
-                          _stream())
+                          *_amax_arg(row_amax, M, (N + 63) // 64), _stream())
     _lib.check(rc, "cdm_gemm_fp8")
     return out
 
@@ -245,8 +277,10 @@ def grouped_gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wqs: Sequence[torch.Ten
                      segments: Sequence[Tuple[int, int]], *, w2qs: Optional[Sequence[torch.Tensor]] = None,
                      sw2s: Optional[Sequence[torch.Tensor]] = None, epilogue: str = "none", residual=None,
                      gates: Optional[Sequence[Optional[torch.Tensor]]] = None, cos=None, sin=None, rope_cols: int = 0,
-                     head_dim: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """e4m3 form of ``grouped_gemm``: ``sa`` [M] per-token scales, ``sws[g]`` / ``sw2s[g]`` per-channel weight scales."""
+                     head_dim: int = 0, out: Optional[torch.Tensor] = None,
+                     row_amax: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """e4m3 form of ``grouped_gemm``: ``sa`` [M] per-token scales, ``sws[g]`` / ``sw2s[g]`` per-channel weight scales;
+    ``row_amax`` as in ``gemm_fp8``."""
     lib = _lib.load()
     M, K = aq.shape
     N = wqs[0].shape[0]
@@ -272,7 +306,7 @@ def grouped_gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wqs: Sequence[torch.Ten
                                   epi, _chk(residual, "residual", odt, 2),
                                   residual.stride(0) if residual is not None else 0, gp,
                                   _f32vec(cos, "cos", M * half), _f32vec(sin, "sin", M * half), int(rope_cols),
-                                  int(head_dim), _stream())
+                                  int(head_dim), *_amax_arg(row_amax, M, (N + 63) // 64), _stream())
     _lib.check(rc, "cdm_grouped_gemm_fp8")
     return out
 
@@ -389,9 +423,11 @@ def attention_pack_kv(k: torch.Tensor, v: torch.Tensor, n_heads: int, head_dim: 
 def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, head_dim: int,
                      out: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                      sin: Optional[torch.Tensor] = None, qk_norm=None, prefix=None,
-                     causal_prefix: int = 0, n_kv_heads: Optional[int] = None) -> torch.Tensor:
+                     causal_prefix: int = 0, n_kv_heads: Optional[int] = None,
+                     row_amax: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Second stage of ``attention``: the ``n`` query rows against the keys packed in ``workspace`` (``n`` tokens),
-    preceded by the keys of ``prefix`` = (images, n_prefix_tokens) if given."""
+    preceded by the keys of ``prefix`` = (images, n_prefix_tokens) if given.  ``row_amax``: optional contiguous
+    [n, n_heads] fp32 that receives the largest |out| of each row within each head (for ``quant_rows_from_parts``)."""
     lib = _lib.load()
     n, d = q.shape[0], n_heads * head_dim
     n_kv_heads = n_heads if n_kv_heads is None else int(n_kv_heads)
@@ -404,6 +440,11 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
         raise ValueError("prefix images are smaller than the workspace of n_prefix tokens")
     if workspace.numel() < attn_workspace_bytes(n, n_kv_heads, head_dim):
         raise ValueError("workspace is smaller than the images of n tokens")
+    amax_ptr = None
+    if row_amax is not None:
+        if row_amax.shape != (n, n_heads) or not row_amax.is_contiguous():
+            raise ValueError("row_amax must be a contiguous [n_tokens, n_heads] fp32 tensor")
+        amax_ptr = _chk(row_amax, "row_amax", torch.float32, 2)
     timer = _ATTN_TIMER
     if timer is not None:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -411,7 +452,7 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
     rc = lib.cdm_attn_fwd_packed_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _f32vec(cos, "cos", n * half),
                                       _f32vec(sin, "sin", n * half), _chk(workspace, "workspace", torch.uint8, 1),
                                       _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, n_kv_heads, head_dim,
-                                      qn, pws, npre, int(causal_prefix), _stream())
+                                      qn, pws, npre, int(causal_prefix), amax_ptr, _stream())
     if timer is not None:
         e1.record()
         timer.append((e0, e1))

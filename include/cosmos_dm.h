@@ -99,6 +99,15 @@ int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, float* s, int64
                             void* stream);
 
 /*
+ * The same quantisation (bit for bit) where the kernel that produced `a` left partial row maxima behind:
+ * parts [rows, n_parts] fp32 (row stride ldp), entry (i, c) = max |a[i, j]| over one range of columns j, the ranges
+ * covering the row (cdm_attn_fwd_packed_bf16 writes one entry per head, the SWIGLU epilogue of the e4m3 GEMM one per 64
+ * output columns).  s[i] = max_c parts[i, c] / 448; the row is read once instead of twice.  n_parts <= 4096.
+ */
+int32_t cdm_quant_rows_from_parts_e4m3(const void* a, int64_t lda, const float* parts, int64_t ldp, int64_t n_parts,
+                                       void* q, float* s, int64_t rows, int64_t cols, void* stream);
+
+/*
  * bf16 linear layer(s) with a fused epilogue - replaces nn.Linear (no bias) of the DM branch:
  * add_q_proj/add_k_proj/add_v_proj (fused as one [3d, d] weight), to_add_out, and the
  * moe_gen gate/up/down projections (parameter names: transformers
@@ -124,13 +133,16 @@ int32_t cdm_gemm_bf16(const void* A, int64_t lda, const void* W, int64_t ldw, co
  * fp8 (e4m3) linear with per-token and per-output-channel scales - the quantised variant:
  *   C[i,j] = sa[i] * sw[j] * sum_k Aq[i,k] Wq[j,k]   (fp32 accumulate) -> bf16, then the epilogue.
  * Aq: [M, K] bytes, Wq: [N, K] bytes (W2q/sw2 for CDM_EPI_SWIGLU).  K % 256 == 0.
+ * row_amax (optional, CDM_EPI_SWIGLU only): [M, amax_ld] fp32, amax_ld >= ceil(N / 64); entry (i, c) receives the largest
+ * |C[i, j]| over columns 64 c .. 64 c + 63 (of the bf16 values stored), for cdm_quant_rows_from_parts_e4m3: the hidden
+ * activations are quantised per token for the down projection without a pass that searches the row maxima.
  */
 int32_t cdm_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const void* Wq, int64_t ldw, const float* sw,
                      const void* W2q, const float* sw2,
                      void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int32_t epilogue,
                      const void* R, int64_t ldr, const float* gate,
                      const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
-                     void* stream);
+                     float* row_amax, int64_t amax_ld, void* stream);
 
 /*
  * Standalone 3-D mRoPE on Q and K in place - replaces apply_rotary_pos_emb with mRoPE tables
@@ -201,6 +213,9 @@ int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk
  *   the denoising step, so they are packed once per prompt and passed here at every step, and the per-step call
  *   carries only the generator tokens.  Cannot be combined with causal_prefix.
  * cdm_attn_pack_kv_bf16 sees K / V heads only (n_kv_heads of them).
+ *   row_amax (optional, 4-byte aligned): [n_tokens, n_heads] fp32; entry (i, h) receives the largest |o| of row i within
+ *   head h (of the bf16 values stored) - the partial row maxima cdm_quant_rows_from_parts_e4m3 takes when the attention
+ *   output is quantised per token for the e4m3 output projection.
  */
 int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                               const float* sin, void* workspace, int64_t workspace_bytes, int64_t n_tokens,
@@ -209,7 +224,7 @@ int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, c
                                  const void* workspace, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
                                  int32_t n_kv_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
                                  const void* prefix_workspace, int64_t n_prefix_tokens, int64_t causal_prefix,
-                                 void* stream);
+                                 float* row_amax, void* stream);
 
 /*
  * cdm_attn_fwd_bf16 for callers that cannot allocate device memory or carry a workspace (code under HIP graph
@@ -256,7 +271,7 @@ int32_t cdm_grouped_gemm_fp8(const void* Aq, int64_t lda, const float* sa, const
                              int64_t N, int64_t K, int32_t epilogue,
                              const void* R, int64_t ldr, const float* const* gate,
                              const float* cos, const float* sin, int64_t rope_cols, int32_t head_dim,
-                             void* stream);
+                             float* row_amax, int64_t amax_ld, void* stream);
 
 /* Exported by the cross-check build only (libcosmos_dm_hip_crosscheck.so, compiled with -DCDM_CROSSCHECK), which the
  * parity tests load to compare the default kernels with their predecessors; the product library has no such state.

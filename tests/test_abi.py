@@ -103,9 +103,9 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
     assert lib.cdm_attn_fwd_bf16(*args, None, 17, None) == _lib.ERR_BAD_ARG                  # causal prefix > n_tokens
     pk = (fake, 64, None, None, fake, fake, 64, 16, 1, 1, 64, None)
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 100, 0, None) == _lib.ERR_BAD_SHAPE       # prefix not whole tiles
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 64, 0, None) == _lib.ERR_BAD_ARG          # prefix size without images
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 64, 4, None) == _lib.ERR_UNSUPPORTED      # prefix images + causal prefix
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 100, 0, None, None) == _lib.ERR_BAD_SHAPE       # prefix not whole tiles
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 64, 0, None, None) == _lib.ERR_BAD_ARG          # prefix size without images
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 64, 4, None, None) == _lib.ERR_UNSUPPORTED      # prefix images + causal prefix
     qn = _lib.QkNorm(fake, fake, ends, 2, 0.0)
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
     # grouped-query attention: the K/V head count must divide the query head count
@@ -113,8 +113,18 @@ def test_bad_arguments_are_rejected_on_the_host():
                                               64 * H, 16, H, Hkv, 64, fake, 1 << 24, None, 0, None)
     assert gq(6, 4) == _lib.ERR_BAD_SHAPE and "divide" in _lib.last_error()
     assert gq(6, 0) == _lib.ERR_BAD_SHAPE
-    assert lib.cdm_attn_fwd_packed_bf16(fake, 384, None, None, fake, fake, 384, 16, 6, 4, 64, None, None, 0, 0,
+    assert lib.cdm_attn_fwd_packed_bf16(fake, 384, None, None, fake, fake, 384, 16, 6, 4, 64, None, None, 0, 0, None,
                                         None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 0, 0, fake + 2, None) == _lib.ERR_BAD_ALIGN       # misaligned row_amax
+    # partial row maxima: only the SwiGLU epilogue of the e4m3 GEMM writes them; the quantiser that reads them checks its table
+    f8 = lambda epi, amax, ld: lib.cdm_gemm_fp8(fake, 256, fake, fake, 256, fake, fake, fake, fake, 256, 8, 256, 256, epi, None, 0,
+                                                None, None, None, 0, 0, amax, ld, None)
+    assert f8(_lib.EPI_NONE, fake, 4) == _lib.ERR_BAD_ARG and "SWIGLU" in _lib.last_error()
+    assert f8(_lib.EPI_SWIGLU, fake, 3) == _lib.ERR_BAD_ARG            # 256 columns need 4 entries per row
+    assert lib.cdm_quant_rows_from_parts_e4m3(fake, 128, None, 4, 4, fake, fake, 4, 128, None) == _lib.ERR_BAD_ARG
+    assert lib.cdm_quant_rows_from_parts_e4m3(fake, 128, fake, 2, 4, fake, fake, 4, 128, None) == _lib.ERR_BAD_ARG
+    assert lib.cdm_quant_rows_from_parts_e4m3(fake, 128, fake, 4, 4, fake, fake, 4, 100, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_quant_rows_from_parts_e4m3(fake, 128, fake, 4, 4, fake, fake, 0, 128, None) in (_lib.OK, _lib.ERR_NO_DEVICE)
     # the workspace holds K/V heads only
     assert lib.cdm_attn_workspace_bytes(100, 2, 64) * 3 == lib.cdm_attn_workspace_bytes(100, 6, 64)
     # QKV projection with fused tile images: head_dim 128 only, segments tile the sequence on 64-token boundaries,

@@ -553,6 +553,53 @@ def test_quant_rows_exact(rows, cols):
     assert torch.equal(q.float().cpu(), wq)
 
 
+@pytest.mark.parametrize("n,H,Hkv,hd", [(300, 4, 2, 128), (1000, 2, 2, 128), (130, 3, 3, 64)])
+def test_quant_from_attention_row_maxima(n, H, Hkv, hd):
+    """The attention kernel leaves the largest |o| of every output row within every head; the quantiser that starts from
+    those partial maxima must give the scales and e4m3 codes of the plain two-pass quantiser bit for bit."""
+    g = gen(5 * n + H)
+    d, dkv = H * hd, Hkv * hd
+    qkv, _ = rand_bf16((n, d + 2 * dkv), g, 1.5)
+    img = ops.attention_pack_kv(qkv[:, d:d + dkv], qkv[:, d + dkv:], Hkv, hd)
+    parts = torch.full((n, H), float("nan"), dtype=torch.float32, device=dev())
+    o = ops.attention_packed(qkv[:, :d], img, H, hd, n_kv_heads=Hkv, row_amax=parts)
+    assert torch.equal(parts, o.float().abs().view(n, H, hd).amax(-1))
+    q_ref, s_ref = ops.quant_rows(o)
+    q, s = ops.quant_rows_from_parts(o, parts)
+    assert torch.equal(s, s_ref) and torch.equal(q.view(torch.uint8), q_ref.view(torch.uint8))
+    o0 = ops.attention_packed(qkv[:, :d], img, H, hd, n_kv_heads=Hkv)        # the maxima are an extra output, nothing else
+    assert torch.equal(o0, o)
+
+
+@pytest.mark.parametrize("M,N,K,split", [(300, 256, 256, 0), (1000, 1096, 512, 0), (700, 512, 256, 256), (64, 64, 256, 0)])
+def test_quant_from_swiglu_row_maxima(M, N, K, split):
+    """The SwiGLU epilogue of the e4m3 GEMM leaves the largest |h| of every row within every 64 output columns (ragged
+    last column block, ragged last row tile, two weight sets); quantising from them equals the two-pass quantiser."""
+    g = gen(M + N + K)
+    a, _ = rand_bf16((M, K), g)
+    segs = [(0, M)] if not split else [(0, split), (split, M - split)]
+    wg = [rand_bf16((N, K), g, 0.1)[0] for _ in segs]
+    wu = [rand_bf16((N, K), g, 0.1)[0] for _ in segs]
+    aq, sa = ops.quant_rows(a)
+    gq, uq = [ops.quant_rows(w) for w in wg], [ops.quant_rows(w) for w in wu]
+    n_parts = (N + 63) // 64
+    parts = torch.full((M, n_parts + 1), float("nan"), dtype=torch.float32, device=dev())     # row stride > n_parts
+    h = ops.grouped_gemm_fp8(aq, sa, [w for w, _ in gq], [s for _, s in gq], segs, w2qs=[w for w, _ in uq],
+                             sw2s=[s for _, s in uq], epilogue="swiglu", row_amax=parts)
+    h0 = ops.grouped_gemm_fp8(aq, sa, [w for w, _ in gq], [s for _, s in gq], segs, w2qs=[w for w, _ in uq],
+                              sw2s=[s for _, s in uq], epilogue="swiglu")
+    assert torch.equal(h, h0)
+    pad = torch.zeros((M, n_parts * 64), dtype=torch.float32, device=dev())
+    pad[:, :N] = h.float().abs()
+    assert torch.equal(parts[:, :n_parts], pad.view(M, n_parts, 64).amax(-1))
+    assert bool(torch.isnan(parts[:, n_parts]).all())                        # nothing beyond the row's entries is touched
+    q_ref, s_ref = ops.quant_rows(h)
+    q, s = ops.quant_rows_from_parts(h, parts[:, :n_parts])
+    assert torch.equal(s, s_ref) and torch.equal(q.view(torch.uint8), q_ref.view(torch.uint8))
+    with pytest.raises(RuntimeError):
+        ops.gemm_fp8(aq, sa, gq[0][0], gq[0][1], row_amax=parts)            # not a SwiGLU epilogue
+
+
 def test_adaln_rmsnorm_quant():
     g = gen(31)
     n, d = 70, 1024
