@@ -279,6 +279,7 @@ struct PackedParams {
     const char* vp_prefix;
     const float* kmax_prefix;
     int n_prefix_tiles;
+    int prefix_last_valid;       // keys of the last prefix tile that exist (1..64; the rest of that tile is zero padding)
     int causal_prefix;           // query rows < causal_prefix see keys <= their own index only; the others see all keys
     bf16_t* o; int64_t ldo;
     float* row_amax;             // optional [n_tokens, n_heads]: largest |o| of each output row within each head (as stored)
@@ -503,7 +504,14 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) s_a[kb][qb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     scores_tile<HD, QB>(sk, qf, s_a, lane);
+    // the padding of a prefix that does not fill its last tile sits in the MIDDLE of the key sequence: that one tile is
+    // masked like a ragged last tile (pre_rag_tile = its index, or -1)
+    const int pre_rag_tile = (NP > 0 && p.prefix_last_valid < BN) ? NP - 1 : -1;
+    int pre_valid[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) pre_valid[qb] = p.prefix_last_valid;
     if (causal_wg || (NT == 1 && ragged)) mask_scores<QB>(s_a, klim, lane);
+    if (pre_rag_tile == 0) mask_scores<QB>(s_a, pre_valid, lane);
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
         const float m0 = tile_row_max<QB>(s_a, qb);      // exact first reference: every row has at least one finite score
@@ -566,11 +574,13 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
         if (!late_sync) { sync(); load_k(); }                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         int nvalid[QB];                                                                                         \
-        _Pragma("unroll") for (int qb = 0; qb < QB; ++qb) nvalid[qb] = klim[qb] - (j + 1) * BN;                 \
+        const bool pre_rag = j + 1 == pre_rag_tile;                                                             \
+        _Pragma("unroll") for (int qb = 0; qb < QB; ++qb)                                                       \
+            nvalid[qb] = pre_rag ? p.prefix_last_valid : klim[qb] - (j + 1) * BN;                               \
         /* does tile j + 1 (the scores block A computes) need row maxima?  its bit of the wave's table */      \
         pipe_step<HD, QB, LATE>([&]() { if (late_sync) { sync(); load_k(); } else load_v(); }, p.late_r,       \
                           sk + ks_next * TILE_BYTES, sv + v_cur * TILE_BYTES, sk + k_next2 * TILE_BYTES, qf, kw, \
-                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || (ragged && j + 2 >= NT), nvalid,   \
+                          SCUR, SNEXT, oacc, negm, l_run, lane, causal_wg || pre_rag || (ragged && j + 2 >= NT), nvalid, \
                           j + 1, next_hot, need_always, hot);     /* tile j + 1: the scores block A computes */ \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         if (late_sync) load_v();                                                                                \
@@ -822,8 +832,8 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     CDM_REQUIRE((reinterpret_cast<uintptr_t>(row_amax) & 3u) == 0, CDM_ERR_BAD_ALIGN, "attn_fwd_packed: row_amax must be 4-byte aligned");
     CDM_REQUIRE(n_kv_heads > 0 && n_heads > 0 && n_heads % n_kv_heads == 0, CDM_ERR_BAD_SHAPE,
                 "attn_fwd_packed: n_kv_heads=%d must divide n_heads=%d", n_kv_heads, n_heads);
-    CDM_REQUIRE(n_prefix_tokens >= 0 && n_prefix_tokens % BN == 0 && n_prefix_tokens < (1ll << 23), CDM_ERR_BAD_SHAPE,
-                "attn_fwd_packed: n_prefix_tokens=%lld must be a non-negative multiple of %d", (long long)n_prefix_tokens, BN);
+    CDM_REQUIRE(n_prefix_tokens >= 0 && n_prefix_tokens < (1ll << 23), CDM_ERR_BAD_SHAPE,
+                "attn_fwd_packed: n_prefix_tokens=%lld out of range", (long long)n_prefix_tokens);
     CDM_REQUIRE((n_prefix_tokens > 0) == (prefix_workspace != nullptr) && cdm_aligned16(prefix_workspace), CDM_ERR_BAD_ARG,
                 "attn_fwd_packed: prefix_workspace and n_prefix_tokens must be given together (16-byte aligned)");
     CDM_REQUIRE(causal_prefix >= 0 && causal_prefix <= n_tokens, CDM_ERR_BAD_ARG,
@@ -848,7 +858,8 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     p.kp_prefix = (const char*)prefix_workspace;
     p.vp_prefix = (const char*)prefix_workspace + image_bytes(n_prefix_tokens, n_kv_heads, head_dim);
     p.kmax_prefix = (const float*)((const char*)prefix_workspace + 2 * image_bytes(n_prefix_tokens, n_kv_heads, head_dim));
-    p.n_prefix_tiles = (int)(n_prefix_tokens / BN);
+    p.n_prefix_tiles = (int)(pad_tokens(n_prefix_tokens) / BN);
+    p.prefix_last_valid = (int)(n_prefix_tokens - (pad_tokens(n_prefix_tokens) - BN));      // BN for whole tiles
     p.causal_prefix = (int)causal_prefix;
     p.o = (bf16_t*)o; p.ldo = ldo;
     p.row_amax = row_amax;

@@ -584,8 +584,8 @@ class DMStack(nn.Module):
         c = self.cfg
         if not c.hybrid_mask:
             raise RuntimeError("context reuse needs the hybrid mask (DMConfig.hybrid_mask)")
-        if c.n_text == 0 or c.n_text % 64:
-            raise ValueError("context reuse needs a text run whose length is a positive multiple of 64")
+        if c.n_text == 0:
+            raise ValueError("context reuse needs a text run")
         x = self._stream(_as2d(encoder_hidden_states))
         if x.shape != (c.n_text, c.d_model):
             raise ValueError(f"context has shape {tuple(x.shape)}, expected {(c.n_text, c.d_model)}")

@@ -208,7 +208,8 @@ int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk
  * attention kernel proper reads Q (rotating it with the same tables) and the workspace.  A caller that
  * times or profiles the attention kernel alone, or that reuses packed K/V across calls, uses these.
  *   prefix_workspace / n_prefix_tokens (optional): tile images, made by an earlier cdm_attn_pack_kv_bf16 call over
- *   n_prefix_tokens tokens (a multiple of 64), of keys that PRECEDE the keys of `workspace`; the n_tokens queries
+ *   n_prefix_tokens tokens (any count: the padding of a last, partial tile is masked), of keys that PRECEDE the keys of
+ *   `workspace`; the n_tokens queries
  *   then attend to n_prefix_tokens + n_tokens keys.  Under the hybrid mask the K/V of the text run do not depend on
  *   the denoising step, so they are packed once per prompt and passed here at every step, and the per-step call
  *   carries only the generator tokens.  Cannot be combined with causal_prefix.

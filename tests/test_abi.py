@@ -103,7 +103,7 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
     assert lib.cdm_attn_fwd_bf16(*args, None, 17, None) == _lib.ERR_BAD_ARG                  # causal prefix > n_tokens
     pk = (fake, 64, None, None, fake, fake, 64, 16, 1, 1, 64, None)
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 100, 0, None, None) == _lib.ERR_BAD_SHAPE       # prefix not whole tiles
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, -64, 0, None, None) == _lib.ERR_BAD_SHAPE       # negative prefix length
     assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 64, 0, None, None) == _lib.ERR_BAD_ARG          # prefix size without images
     assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 64, 4, None, None) == _lib.ERR_UNSUPPORTED      # prefix images + causal prefix
     qn = _lib.QkNorm(fake, fake, ends, 2, 0.0)

@@ -358,13 +358,15 @@ def test_transformer_with_stack_edges_and_loaded_checkpoint(tmp_path):
     assert_close(out["action"][0], want_act, BF16_COS, BF16_REL, "action head")
 
 
-@pytest.mark.parametrize("n_kv_heads", [None, 1])
-def test_hybrid_mask_stack_and_context_reuse(n_kv_heads):
+@pytest.mark.parametrize("n_kv_heads,P", [(None, 64), (1, 64), (None, 70), (1, 37)])
+def test_hybrid_mask_stack_and_context_reuse(n_kv_heads, P):
     """Two-branch stack under the hybrid mask: (1) joint forward vs the masked fp32 oracle; (2) the text run's K/V
     packed once per prompt and reused: same video output from a forward that carries only the generator tokens;
     (3) the reused cache stays valid for another timestep.  Also with one K/V head for the two query heads (the kept
-    images then hold K/V heads only)."""
-    cfg = DMConfig("hyb", 256, 2, 128, 512, 2, (2, 5, 8), n_text=64, n_action=7, n_branches=3, qk_norm=True,
+    images then hold K/V heads only), and with text runs that do not fill their last 64-key tile (70, 37 tokens: the joint
+    forward then takes the GEMM + re-tiling pair for the segments off a tile boundary, the cached forward masks the padding
+    of the prefix images)."""
+    cfg = DMConfig("hyb", 256, 2, 128, 512, 2, (2, 5, 8), n_text=P, n_action=7, n_branches=3, qk_norm=True,
                    hybrid_mask=True, n_kv_heads=n_kv_heads)
     st = DMStack(cfg, device=dev())
     st.reset_parameters(41)
@@ -376,7 +378,7 @@ def test_hybrid_mask_stack_and_context_reuse(n_kv_heads):
             blk.adaLN_modulation.bias.copy_(0.2 * torch.randn(blk.adaLN_modulation.bias.shape, generator=g, device=dev()))
     gc = torch.Generator().manual_seed(42)
     xv, xvr = rand_bf16((1, cfg.n_video, 256), gc)
-    xt, xtr = rand_bf16((1, 64, 256), gc)
+    xt, xtr = rand_bf16((1, P, 256), gc)
     xa, xar = rand_bf16((1, 7, 256), gc)
     t = torch.tensor([333.0])
     out = st(xv, t.to(dev()), encoder_hidden_states=xt, action_states=xa, return_dict=True)
@@ -384,18 +386,18 @@ def test_hybrid_mask_stack_and_context_reuse(n_kv_heads):
     f = lambda p: p.detach().float().cpu()
     c = O.time_mlp(O.timestep_embedding(t), f(te.linear_1.weight), f(te.linear_1.bias), f(te.linear_2.weight), f(te.linear_2.bias))
     mods = [O.adaln_modulation(c, f(b.adaLN_modulation.weight), f(b.adaLN_modulation.bias)) for b in st.blocks]
-    pos = O.joint_positions([("text", 64), ("video", cfg.grid), ("action", 7)])
+    pos = O.joint_positions([("text", P), ("video", cfg.grid), ("action", 7)])
     cos, sin = O.mrope_cos_sin(pos, 128, cfg.mrope_sections)
     x0 = torch.cat([xtr[0], xvr[0], xar[0]])
-    want = O.dm_stack(x0, [oracle_weights(b, 3) for b in st.blocks], mods, cos, sin, 2, st.segments(), causal_prefix=64)
+    want = O.dm_stack(x0, [oracle_weights(b, 3) for b in st.blocks], mods, cos, sin, 2, st.segments(), causal_prefix=P)
     assert_close(out["joint"], want, BF16_COS, BF16_REL, "hybrid-mask stack (joint)")
     want_full = O.dm_stack(x0, [oracle_weights(b, 3) for b in st.blocks], mods, cos, sin, 2, st.segments())
-    assert O.max_rel_err(want[:64], want_full[:64]) > 1e-2           # the mask is live
+    assert O.max_rel_err(want[:P], want_full[:P]) > 1e-2           # the mask is live
     # (2) context reuse
     cache = st.precompute_context(xt)
     out2 = st(xv, t.to(dev()), action_states=xa, return_dict=True, context_cache=cache)
     assert_close(out2["sample"][0], out["sample"][0].float().cpu(), 0.99999, 4e-3, "cached context == joint forward")
-    assert_close(out2["sample"][0], want[64:64 + cfg.n_video], BF16_COS, BF16_REL, "cached context vs oracle")
+    assert_close(out2["sample"][0], want[P:P + cfg.n_video], BF16_COS, BF16_REL, "cached context vs oracle")
     # (3) another timestep with the same cache
     t2 = torch.tensor([871.0])
     out3 = st(xv, t2.to(dev()), action_states=xa, return_dict=True, context_cache=cache)

@@ -443,10 +443,12 @@ def test_attention_grouped_query(n, H, Hkv, hd, P, variant, request):
         assert torch.equal(o, o2)
 
 
-@pytest.mark.parametrize("P,m,H,hd", [(64, 200, 2, 128), (128, 65, 1, 64), (512, 700, 1, 128)])
+@pytest.mark.parametrize("P,m,H,hd", [(64, 200, 2, 128), (128, 65, 1, 64), (512, 700, 1, 128), (100, 300, 2, 128), (1, 70, 1, 64),
+                                      (65, 64, 1, 128), (500, 1000, 1, 128)])
 def test_attention_with_prefix_key_images(P, m, H, hd):
     """Keys packed once (the text run) and prepended to the per-call keys: the m query rows must equal rows P.. of
-    full attention over all P + m tokens; mRoPE and QK-norm in registers on both sides."""
+    full attention over all P + m tokens; mRoPE and QK-norm in registers on both sides.  A prefix that does not fill
+    its last 64-key tile (100, 1, 65, 500 tokens) leaves padding in the middle of the key sequence, which is masked."""
     g = gen(P + m)
     n, d = P + m, H * hd
     pos, _ = rotary.build_positions(n, (0, 0, 0), 0)
