@@ -56,7 +56,9 @@ SIGNATURES = {
     "cdm_attn_static_scratch_bytes": (_I64, []),
     "cdm_attn_fwd_static_bf16": (_I32, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _I64, _P]),
     "cdm_attn_pack_kv_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _P]),
-    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _P, _I64, _I64, _P, _P]),
+    "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _P, _I64, _I64, _P, _P,
+                                        _I64, _P]),
+    "cdm_attn_split_scratch_bytes": (_I64, [_I64, _I32, _I32]),
     "cdm_grouped_gemm_fp8": (_I32, [_P, _I64, _P, C.POINTER(_P), C.POINTER(_P), _I64, C.POINTER(_P), C.POINTER(_P), _P, _I64,
                                     C.POINTER(_I64), C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P,
                                     _P, _I64, _I32, _P, _I64, _P]),

@@ -290,6 +290,12 @@ struct PackedParams {
     int always_max;              // cross-check: take the row maxima of every tile whatever the norm bound says
     float scale_log2e;           // factor on Q ahead of its rounding to bf16: log2(e)/sqrt(HD), or only its power of two
     float late_r;                // ... with the rest of it (in [1, 2)) applied to the fp32 scores (LATE kernels)
+    // Split of the last, partial round of workgroups (see SplitPlan): the last `split_tail` workgroups of every XCD
+    // are replaced by `split` units each, which cover consecutive ranges of the key tiles and leave a normalised partial
+    // output and the row's log-sum in scratch memory for merge_split_kernel.  split = 1: no split.
+    int split, split_tail;
+    bf16_t* part_o;              // [8 * split_tail * split][256][HD]
+    float* part_lse;             // [8 * split_tail * split][256]   log2 of the unit's sum of exponentials, reference added
 };
 
 // QS = query sub-tiles (of 32 rows = two 16-row blocks) per wave: QS = 1 -> 8 waves, two per SIMD, 256 registers each;
@@ -303,6 +309,7 @@ constexpr float kSafeLog2 = 60.0f;      // largest excess over the reference tha
 // and the fp32 scores by the rest, one multiplication per score; calls that rotate or normalise Q round it once anyway
 // and fold the whole factor into that rounding.
 constexpr int kMaxKm = 2048;            // key tiles that get a decision of their own (131,072 keys); longer sequences: one per head
+constexpr int kMaxSplit = 8;            // most key ranges a query block of the last round is split into
 
 template <int HD, int QS, bool LATE>
 __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS, 2 / QS))) void attn_fwd_pipe_kernel(
@@ -327,10 +334,23 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // ONE XCD, so a head's K / V tile images are fetched into one L2 instead of eight, and an XCD owns a contiguous
     // range of heads, so the query heads that share a K / V head (grouped-query attention) share an L2 as well.
     int head, qblk;
+    int unit = -1, part = 0;      // split unit: index into the scratch arrays, and which range of the key tiles
     {
         const int nqb = p.n_qblocks, nh = p.n_heads;
-        const int xcd = blockIdx.x & 7, k = blockIdx.x >> 3;      // k-th workgroup of its XCD
+        const int xcd = blockIdx.x & 7;
+        int k = blockIdx.x >> 3;                                  // k-th workgroup of its XCD
         const int hpx = (nh + 7) >> 3;                            // heads per XCD (the last XCDs may own fewer)
+        if (p.split > 1) {
+            // the last split_tail query blocks of the XCD come `split` times, ordered by key range first: units that run
+            // side by side then stream the same tiles of the same head
+            const int whole = hpx * nqb - p.split_tail;
+            if (k >= whole) {
+                const int u = k - whole;
+                part = u / p.split_tail;
+                k = whole + (u - part * p.split_tail);
+                unit = xcd * p.split_tail * p.split + u;
+            }
+        }
         const int hi = k / nqb;
         head = xcd * hpx + hi;
         qblk = k - hi * nqb;
@@ -348,18 +368,23 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // register, and keeps the index of the next such tile in a scalar register: a step compares its tile index with it
     // (one scalar instruction) and looks the following one up only after a hit.
     // A sequence of more than kMaxKm tiles falls back to one bound per head (kmax_all).
-    const int NP = p.n_prefix_tiles, NM = (p.n_tokens + BN - 1) / BN;
-    const int NT = NP + NM;
+    // A split unit works in a frame of its own: tile 0 is the first tile of its range [t0, t0 + NT), the prefix tiles
+    // are the first NP of that frame (NP <= 0: none left), per-row key limits count from the frame's first key.
+    const int NM = (p.n_tokens + BN - 1) / BN;
+    const int NT_all = p.n_prefix_tiles + NM;
+    const int t0 = unit < 0 ? 0 : (int)((int64_t)NT_all * part / p.split);
+    const int t1 = unit < 0 ? NT_all : (int)((int64_t)NT_all * (part + 1) / p.split);
+    const int NP = p.n_prefix_tiles - t0;
+    const int NT = t1 - t0;
     const bool per_tile = NT <= kMaxKm;
     float kmax_all = 0.0f;
     {
-        const float* km = p.kmax + (int64_t)kv_head * NM;
-        const float* kmp = p.kmax_prefix + (int64_t)kv_head * NP;
+        const float* km = p.kmax + (int64_t)kv_head * NM - p.n_prefix_tiles + t0;      // indexed by the frame's tile number
+        const float* kmp = p.kmax_prefix + (int64_t)kv_head * p.n_prefix_tiles + t0;
         if (per_tile) {
-            for (int i = threadIdx.x; i < kMaxKm; i += 512 / QS) s_km[i] = i >= NT ? 0.0f : (i < NP ? kmp[i] : km[i - NP]);
+            for (int i = threadIdx.x; i < kMaxKm; i += 512 / QS) s_km[i] = i >= NT ? 0.0f : (i < NP ? kmp[i] : km[i]);
         } else {
-            for (int i = lane; i < NM; i += 64) kmax_all = fmaxf(kmax_all, km[i]);
-            for (int i = lane; i < NP; i += 64) kmax_all = fmaxf(kmax_all, kmp[i]);
+            for (int i = lane; i < NT; i += 64) kmax_all = fmaxf(kmax_all, i < NP ? kmp[i] : km[i]);
             kmax_all = wave_max(kmax_all);
         }
     }
@@ -453,7 +478,8 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     }
 
     // key tiles: NP whole tiles of the prefix images, then the NM tiles of the main images
-    const int n_keys = NP * BN + p.n_tokens;
+    // keys of the frame: a range that ends ahead of the sequence's last tile ends on a full tile
+    const int n_keys = t1 < NT_all ? NT * BN : p.n_prefix_tiles * BN + p.n_tokens - t0 * BN;
     const int last_valid = n_keys - (NT - 1) * BN;
     // per-row key limit and the tiles this workgroup needs: a query block inside the causal prefix stops at its
     // own last row, and every tile it visits is masked per row
@@ -472,8 +498,8 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     // base + t * TILE_BYTES with base shifted back by the prefix length: one 32-bit offset serves both
     const char* kbase = p.kp + ((int64_t)kv_head * NM - NP) * TILE_BYTES;
     const char* vbase = p.vp + ((int64_t)kv_head * NM - NP) * TILE_BYTES;
-    const char* kpre = p.kp_prefix + (int64_t)kv_head * NP * TILE_BYTES;
-    const char* vpre = p.vp_prefix + (int64_t)kv_head * NP * TILE_BYTES;
+    const char* kpre = p.kp_prefix + ((int64_t)kv_head * p.n_prefix_tiles + t0) * TILE_BYTES;
+    const char* vpre = p.vp_prefix + ((int64_t)kv_head * p.n_prefix_tiles + t0) * TILE_BYTES;
     const uint32_t sk_addr = lds_addr_of(sk) + wave * 1024, sv_addr = lds_addr_of(sv) + wave * 1024;
 
     // tile `t` (clamped to the last tile, so that every step issues the same number of loads and the
@@ -614,7 +640,9 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             *reinterpret_cast<uint2*>(stage + (qb * 16 + r16) * PITCH + (16 * hb + 4 * g4) * 2) = w;
             amax = fmaxf(fmaxf(amax, fmaxf(fabsf(bf16lo(w.x)), fabsf(bf16hi(w.x)))), fmaxf(fabsf(bf16lo(w.y)), fabsf(bf16hi(w.y))));
         }
-        if (p.row_amax != nullptr) {      // the row's channels of this head are spread over the four quarter-waves
+        if (unit >= 0) {      // a split unit leaves log2 of its sum of exponentials (reference added back) beside its rows
+            if (g4 == 0) p.part_lse[(int64_t)unit * BMQ + wave * (32 * QS) + qb * 16 + r16] = __log2f(l_tot) - negm[qb][0];
+        } else if (p.row_amax != nullptr) {      // the row's channels of this head are spread over the four quarter-waves
             amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
             amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
             const int qrow = q0 + qb * 16 + r16;
@@ -624,12 +652,62 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
     constexpr int LPR = HD / 8, RPI = 64 / LPR;             // lanes per row, rows per store instruction
     const int rl = lane / LPR, ch = lane % LPR;
+    bf16_t* orow = unit < 0 ? p.o + (int64_t)q0 * p.ldo + head * HD
+                            : p.part_o + ((int64_t)unit * BMQ + wave * (32 * QS)) * HD;      // row of the wave's first query
+    const int64_t ldo = unit < 0 ? p.ldo : HD;
 #pragma unroll
     for (int it = 0; it < 32 * QS / RPI; ++it) {
         const int rloc = it * RPI + rl;
         const uint4 v = *reinterpret_cast<const uint4*>(stage + rloc * PITCH + ch * 16);
-        const int qrow = q0 + rloc;
-        if (qrow < p.n_tokens) *reinterpret_cast<uint4*>(p.o + (int64_t)qrow * p.ldo + head * HD + ch * 8) = v;
+        if (q0 + rloc < p.n_tokens) *reinterpret_cast<uint4*>(orow + rloc * ldo + ch * 8) = v;
+    }
+}
+
+// Merge of the split units' partial results: one workgroup per query block of the split tail.  Part i of a row holds
+// o_i = (sum_k p_k v_k) / l_i over its key range and lse_i = log2(l_i) + m_i; the row of the whole range is
+// sum_i w_i o_i / sum_i w_i with w_i = 2^(lse_i - max_i lse_i).
+template <int HD>
+__global__ __launch_bounds__(256) void merge_split_kernel(const PackedParams p) {
+    constexpr int LPR = HD / 8;                       // lanes per row: 16 bytes each
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;      // j-th query block of the XCD's tail
+    const int nqb = p.n_qblocks, hpx = (p.n_heads + 7) >> 3;
+    const int k = hpx * nqb - p.split_tail + j;
+    const int hi = k / nqb, head = xcd * hpx + hi, qblk = k - hi * nqb;
+    for (int idx = threadIdx.x; idx < BMQ * LPR; idx += 256) {
+        const int r = idx / LPR, ch = idx % LPR;
+        const int qrow = qblk * BMQ + r;
+        float lse[kMaxSplit], mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < kMaxSplit; ++i) {
+            lse[i] = i < p.split ? p.part_lse[((int64_t)xcd * p.split_tail * p.split + i * p.split_tail + j) * BMQ + r] : -INFINITY;
+            mx = fmaxf(mx, lse[i]);
+        }
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, den = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kMaxSplit; ++i) {
+            if (i >= p.split) break;
+            const float w = exp2f(lse[i] - mx);
+            den += w;
+            const uint4 u = *reinterpret_cast<const uint4*>(
+                p.part_o + (((int64_t)xcd * p.split_tail * p.split + i * p.split_tail + j) * BMQ + r) * HD + ch * 8);
+            const uint32_t q[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { acc[2 * e] += w * bf16lo(q[e]); acc[2 * e + 1] += w * bf16hi(q[e]); }
+        }
+        const float inv = 1.0f / den;
+        uint4 o;
+        o.x = pack_bf16x2(acc[0] * inv, acc[1] * inv); o.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
+        o.z = pack_bf16x2(acc[4] * inv, acc[5] * inv); o.w = pack_bf16x2(acc[6] * inv, acc[7] * inv);
+        if (qrow < p.n_tokens) *reinterpret_cast<uint4*>(p.o + (int64_t)qrow * p.ldo + head * HD + ch * 8) = o;
+        if (p.row_amax != nullptr) {      // LPR consecutive lanes hold the row
+            const uint32_t q[4] = {o.x, o.y, o.z, o.w};
+            float amax = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) amax = fmaxf(amax, fmaxf(fabsf(bf16lo(q[e])), fabsf(bf16hi(q[e]))));
+#pragma unroll
+            for (int off = 1; off < LPR; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            if (ch == 0 && qrow < p.n_tokens) p.row_amax[(int64_t)qrow * p.n_heads + head] = amax;
+        }
     }
 }
 
@@ -750,6 +828,35 @@ inline int64_t kmax_bytes(int64_t n_tokens, int n_heads) {      // one float per
     return (pad_tokens(n_tokens) / BN * n_heads * 4 + 15) / 16 * 16;
 }
 
+// The last, partial round of workgroups.  An XCD owns heads/8 x query blocks workgroups and runs 32 at a time (one per
+// CU: the K / V rings fill the LDS), so a launch takes ceil(workgroups / 32) rounds of equal length however few
+// workgroups the last round holds.  The plan cuts each query block of that last round into `split` units by key range
+// (the smallest of 2, 4, 8 that minimises ceil(tail * split / 32) / split rounds), which the merge kernel puts together.
+// Only where it pays: the chip is power-limited, so a round that leaves CUs idle already runs faster than a full one,
+// and every unit repeats the set-up; measured at 56 k tokens x 32 heads, a plan that ends in half a round or less gains
+// 1 - 3 % and one that ends in three quarters gains nothing.  So: the split round must take at most half a round, and
+// there must be at least two whole rounds, heads a multiple of 8, at least 8 key tiles per unit, and no causal rows in
+// the tail's query blocks.
+struct SplitPlan { int split, tail; int64_t bytes; };
+inline SplitPlan split_plan(int64_t n_tokens, int n_heads, int head_dim, int64_t causal_prefix) {
+    SplitPlan none{1, 0, 0};
+    const int64_t nqb = (n_tokens + BMQ - 1) / BMQ, per_xcd = (n_heads / 8) * nqb;
+    if (n_heads % 8 != 0 || per_xcd < 64) return none;
+    const int tail = (int)(per_xcd % 32);
+    if (tail == 0) return none;
+    if (causal_prefix > 0 && (tail >= nqb || (nqb - tail) * BMQ < causal_prefix)) return none;
+    const int64_t nm = (n_tokens + BN - 1) / BN;
+    int best = 1;
+    double best_cost = 1.0;
+    for (int s = 2; s <= kMaxSplit && nm / s >= 8; s *= 2) {
+        const double cost = (double)((tail * s + 31) / 32) / s;
+        if (cost < best_cost - 1e-9) { best_cost = cost; best = s; }
+    }
+    if (best == 1 || best_cost > 0.5 + 1e-9) return none;
+    const int64_t units = 8ll * tail * best;
+    return SplitPlan{best, tail, units * BMQ * ((int64_t)head_dim * 2 + 4)};
+}
+
 // host view of the optional QK-norm argument -> kernel descriptor (which = 0: q weights, 1: k weights)
 int32_t make_qk_norm(const char* who, const cdm_qk_norm* qn, int which, int64_t n_tokens, QkNormDev* out) {
     out->w = nullptr; out->n_seg = 0; out->eps = 0.0f;
@@ -790,6 +897,12 @@ extern "C" int64_t cdm_attn_workspace_bytes(int64_t n_tokens, int32_t n_heads, i
     return 2 * image_bytes(n_tokens, n_heads, head_dim) + kmax_bytes(n_tokens, n_heads);
 }
 
+// scratch for the split of the last round of workgroups (0: this shape has nothing to split); n_heads counts QUERY heads
+extern "C" int64_t cdm_attn_split_scratch_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim) {
+    if (n_tokens <= 0 || n_heads <= 0 || (head_dim != 64 && head_dim != 128)) return 0;
+    return split_plan(n_tokens, n_heads, head_dim, 0).bytes;
+}
+
 extern "C" int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                                          const float* sin, void* workspace, int64_t workspace_bytes,
                                          int64_t n_tokens, int32_t n_heads, int32_t head_dim,
@@ -827,8 +940,10 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
                                             int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
                                             const cdm_qk_norm* qk_norm, const void* prefix_workspace,
                                             int64_t n_prefix_tokens, int64_t causal_prefix, float* row_amax,
-                                            void* stream) {
+                                            void* split_scratch, int64_t split_scratch_bytes, void* stream) {
     CDM_REQUIRE(q && workspace && o, CDM_ERR_BAD_ARG, "attn_fwd_packed: null pointer");
+    CDM_REQUIRE(cdm_aligned16(split_scratch) && (split_scratch == nullptr || split_scratch_bytes >= 0), CDM_ERR_BAD_ARG,
+                "attn_fwd_packed: split_scratch must be 16-byte aligned, its size non-negative");
     CDM_REQUIRE((reinterpret_cast<uintptr_t>(row_amax) & 3u) == 0, CDM_ERR_BAD_ALIGN, "attn_fwd_packed: row_amax must be 4-byte aligned");
     CDM_REQUIRE(n_kv_heads > 0 && n_heads > 0 && n_heads % n_kv_heads == 0, CDM_ERR_BAD_SHAPE,
                 "attn_fwd_packed: n_kv_heads=%d must divide n_heads=%d", n_kv_heads, n_heads);
@@ -875,14 +990,22 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
     p.late_r = late ? 2.0f * mant : 1.0f;
     p.n_qblocks = (int)((n_tokens + BMQ - 1) / BMQ);
     // 1-D grid of 8 x ceil(heads / 8) x query blocks ids: id % 8 = XCD, see the kernel's placement rule
-    const int64_t nwg = 8ll * ((n_heads + 7) / 8) * p.n_qblocks;
-    CDM_REQUIRE(nwg < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd_packed: grid too large");
-    dim3 grid((unsigned)nwg);
-    hipStream_t st = (hipStream_t)stream;
     // variant 0 = 32 query rows per wave (8 waves, two per SIMD), row maxima dropped where the norm bound allows;
     // cross-check build only: 1 = 64 query rows per wave (4 waves), 2 = variant 0 with the row maxima always taken
     const int variant = cdm_get_variant(0);
     p.always_max = variant == 2;
+    // the last round's query blocks by key range, if the caller brought the scratch memory for it
+    p.split = 1; p.split_tail = 0; p.part_o = nullptr; p.part_lse = nullptr;
+    const SplitPlan plan = split_plan(n_tokens, n_heads, head_dim, causal_prefix);
+    if (split_scratch != nullptr && plan.split > 1 && split_scratch_bytes >= plan.bytes && variant != 1) {
+        p.split = plan.split; p.split_tail = plan.tail;
+        p.part_o = (bf16_t*)split_scratch;
+        p.part_lse = (float*)((char*)split_scratch + 8ll * plan.tail * plan.split * BMQ * head_dim * 2);
+    }
+    const int64_t nwg = 8ll * ((n_heads + 7) / 8) * p.n_qblocks + 8ll * p.split_tail * (p.split - 1);
+    CDM_REQUIRE(nwg < (1ll << 31), CDM_ERR_BAD_SHAPE, "attn_fwd_packed: grid too large");
+    dim3 grid((unsigned)nwg);
+    hipStream_t st = (hipStream_t)stream;
 #define CDM_ATTN_LAUNCH(QS_, THREADS)                                                                      \
     if (head_dim == 128 && late) attn_fwd_pipe_kernel<128, QS_, true><<<grid, THREADS, 0, st>>>(p);       \
     else if (head_dim == 128) attn_fwd_pipe_kernel<128, QS_, false><<<grid, THREADS, 0, st>>>(p);         \
@@ -894,6 +1017,11 @@ extern "C" int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const fl
 #endif
     { CDM_ATTN_LAUNCH(1, 512); }
 #undef CDM_ATTN_LAUNCH
+    if (p.split > 1) {
+        if ((rc = cdm_check_launch("attn_fwd_packed"))) return rc;
+        if (head_dim == 128) merge_split_kernel<128><<<dim3(8u * p.split_tail), 256, 0, st>>>(p);
+        else merge_split_kernel<64><<<dim3(8u * p.split_tail), 256, 0, st>>>(p);
+    }
     return cdm_check_launch("attn_fwd_packed");
 }
 
@@ -927,8 +1055,11 @@ extern "C" int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, 
     if ((rc = cdm_attn_pack_kv_bf16(k, ldk, v, ldv, cos, sin, workspace, workspace_bytes, n_tokens, n_kv_heads, head_dim,
                                     qk_norm, stream)))
         return rc;
+    // what the caller's workspace holds beyond the images serves the split of the last round
+    const int64_t used = (need + 255) / 256 * 256;
+    void* extra = workspace_bytes > used ? (char*)workspace + used : nullptr;
     return cdm_attn_fwd_packed_bf16(q, ldq, cos, sin, workspace, o, ldo, n_tokens, n_heads, n_kv_heads, head_dim, qk_norm,
-                                    nullptr, 0, causal_prefix, nullptr, stream);
+                                    nullptr, 0, causal_prefix, nullptr, extra, extra ? workspace_bytes - used : 0, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -993,6 +1124,7 @@ extern "C" int32_t cdm_attn_fwd_static_bf16(const void* q, int64_t ldq, const vo
         if (rc) return rc;
         if ((rc = static_scratch(&ws))) return rc;
     }
+    // exactly the images' size: the array holds no scratch for a split of the last round of workgroups
     return cdm_attn_fwd_bf16(q, ldq, k, ldk, v, ldv, cos, sin, o, ldo, n_tokens, n_heads, n_kv_heads, head_dim, ws,
-                             kStaticScratchBytes, qk_norm, causal_prefix, stream);
+                             need, qk_norm, causal_prefix, stream);
 }

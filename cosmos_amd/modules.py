@@ -80,7 +80,8 @@ class Workspace:
         self.qkv = torch.empty((n, d + 2 * n_kv_heads * head_dim), **bf)       # [Q | K | V] columns
         self.attn_out = torch.empty((n, d), **bf)
         self.h = torch.empty((n, hidden), **bf)
-        self.attn_ws = torch.empty((max(ops.attn_workspace_bytes(n, n_kv_heads, head_dim), 16),), dtype=torch.uint8,
+        # K / V tile images, then the scratch with which the attention kernel splits its last round of workgroups
+        self.attn_ws = torch.empty((ops.attn_workspace_total_bytes(n, n_heads, n_kv_heads, head_dim),), dtype=torch.uint8,
                                    device=device)
 
     def fits(self, n: int, d: int, hidden: int, fp8: bool = False) -> bool:
@@ -159,8 +160,8 @@ class DMAttnProcessor:
         elif (self.rope == "in_attention" and self.fuse_kv_pack
               and ops.qkv_pack_applies([(s0, ln) for (s0, ln, _, _) in modality_segments], attn.head_dim)):
             if wsb is None:
-                wsb = torch.empty((ops.attn_workspace_bytes(n, attn.n_kv_heads, attn.head_dim),), dtype=torch.uint8,
-                                  device=x.device)
+                wsb = torch.empty((ops.attn_workspace_total_bytes(n, attn.n_heads, attn.n_kv_heads, attn.head_dim),),
+                                  dtype=torch.uint8, device=x.device)
             attn._qkv_pack(x, quant_scale, modality_segments, qkv, wsb, cos, sin, qkn)
             o_amax = ws.o_amax if (attn.fp8 and ws is not None and ws.fp8) else None
             ops.attention_packed(q, wsb, attn.n_heads, attn.head_dim, o, cos, sin, qkn, prefix, causal_prefix,

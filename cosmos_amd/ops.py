@@ -385,6 +385,24 @@ def attn_workspace_bytes(n_tokens: int, n_kv_heads: int, head_dim: int) -> int:
     return int(_lib.load().cdm_attn_workspace_bytes(n_tokens, n_kv_heads, head_dim))
 
 
+def attn_workspace_total_bytes(n_tokens: int, n_heads: int, n_kv_heads: int, head_dim: int) -> int:
+    """Tile images (rounded up to 256 bytes) plus the scratch of the split: the workspace ``attention`` allocates."""
+    need = attn_workspace_bytes(n_tokens, n_kv_heads, head_dim)
+    return max((need + 255) // 256 * 256 + attn_split_scratch_bytes(n_tokens, n_heads, head_dim), 16)
+
+
+def attn_split_scratch_bytes(n_tokens: int, n_heads: int, head_dim: int) -> int:
+    """Bytes of scratch with which ``attention_packed`` splits the last, partial round of its workgroups by key range
+    (0: nothing to split for this shape).  ``n_heads`` counts query heads."""
+    return int(_lib.load().cdm_attn_split_scratch_bytes(n_tokens, n_heads, head_dim))
+
+
+def _extra_of(workspace: torch.Tensor, need: int) -> Optional[torch.Tensor]:
+    """What a workspace holds beyond the tile images (rounded up to 256 bytes), or None."""
+    used = (need + 255) // 256 * 256
+    return workspace[used:] if workspace.numel() > used else None
+
+
 def _qk_norm_arg(qk_norm, head_dim: int):
     """-> (pointer or None, keep-alive objects) for the optional ``cdm_qk_norm`` argument."""
     if qk_norm is None:
@@ -424,10 +442,13 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
                      out: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                      sin: Optional[torch.Tensor] = None, qk_norm=None, prefix=None,
                      causal_prefix: int = 0, n_kv_heads: Optional[int] = None,
-                     row_amax: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     row_amax: Optional[torch.Tensor] = None,
+                     split_scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Second stage of ``attention``: the ``n`` query rows against the keys packed in ``workspace`` (``n`` tokens),
     preceded by the keys of ``prefix`` = (images, n_prefix_tokens) if given.  ``row_amax``: optional contiguous
-    [n, n_heads] fp32 that receives the largest |out| of each row within each head (for ``quant_rows_from_parts``)."""
+    [n, n_heads] fp32 that receives the largest |out| of each row within each head (for ``quant_rows_from_parts``).
+    ``split_scratch``: optional uint8 buffer of ``attn_split_scratch_bytes`` bytes; default: what ``workspace`` holds
+    beyond the images."""
     lib = _lib.load()
     n, d = q.shape[0], n_heads * head_dim
     n_kv_heads = n_heads if n_kv_heads is None else int(n_kv_heads)
@@ -445,6 +466,10 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
         if row_amax.shape != (n, n_heads) or not row_amax.is_contiguous():
             raise ValueError("row_amax must be a contiguous [n_tokens, n_heads] fp32 tensor")
         amax_ptr = _chk(row_amax, "row_amax", torch.float32, 2)
+    if split_scratch is None:
+        split_scratch = _extra_of(workspace, attn_workspace_bytes(n, n_kv_heads, head_dim))
+    ss_ptr = None if split_scratch is None else _chk(split_scratch, "split_scratch", torch.uint8, 1)
+    ss_bytes = 0 if split_scratch is None else split_scratch.numel()
     timer = _ATTN_TIMER
     if timer is not None:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -452,7 +477,7 @@ def attention_packed(q: torch.Tensor, workspace: torch.Tensor, n_heads: int, hea
     rc = lib.cdm_attn_fwd_packed_bf16(_chk(q, "q", torch.bfloat16, 2), q.stride(0), _f32vec(cos, "cos", n * half),
                                       _f32vec(sin, "sin", n * half), _chk(workspace, "workspace", torch.uint8, 1),
                                       _chk(out, "out", torch.bfloat16, 2), out.stride(0), n, n_heads, n_kv_heads, head_dim,
-                                      qn, pws, npre, int(causal_prefix), amax_ptr, _stream())
+                                      qn, pws, npre, int(causal_prefix), amax_ptr, ss_ptr, ss_bytes, _stream())
     if timer is not None:
         e1.record()
         timer.append((e0, e1))
@@ -482,7 +507,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads: int, h
         out = torch.empty((n, d), dtype=torch.bfloat16, device=q.device)
     need = attn_workspace_bytes(n, n_kv_heads, head_dim)
     if workspace is None:
-        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+        workspace = torch.empty((attn_workspace_total_bytes(n, n_heads, n_kv_heads, head_dim),), dtype=torch.uint8,
+                                device=q.device)
     if _ATTN_TIMER is None and _OP_TIMER is None and prefix is None:
         half = head_dim // 2
         qn, _keep = _qk_norm_arg(qk_norm, head_dim)

@@ -217,6 +217,7 @@ int32_t cdm_attn_fwd_bf16(const void* q, int64_t ldq, const void* k, int64_t ldk
  *   row_amax (optional, 4-byte aligned): [n_tokens, n_heads] fp32; entry (i, h) receives the largest |o| of row i within
  *   head h (of the bf16 values stored) - the partial row maxima cdm_quant_rows_from_parts_e4m3 takes when the attention
  *   output is quantised per token for the e4m3 output projection.
+ *   split_scratch / split_scratch_bytes (optional): see cdm_attn_split_scratch_bytes below; null or too small = one pass.
  */
 int32_t cdm_attn_pack_kv_bf16(const void* k, int64_t ldk, const void* v, int64_t ldv, const float* cos,
                               const float* sin, void* workspace, int64_t workspace_bytes, int64_t n_tokens,
@@ -225,7 +226,20 @@ int32_t cdm_attn_fwd_packed_bf16(const void* q, int64_t ldq, const float* cos, c
                                  const void* workspace, void* o, int64_t ldo, int64_t n_tokens, int32_t n_heads,
                                  int32_t n_kv_heads, int32_t head_dim, const cdm_qk_norm* qk_norm,
                                  const void* prefix_workspace, int64_t n_prefix_tokens, int64_t causal_prefix,
-                                 float* row_amax, void* stream);
+                                 float* row_amax, void* split_scratch, int64_t split_scratch_bytes, void* stream);
+/*
+ * Scratch memory for splitting the last, partial round of attention workgroups (no counterpart in the reference: a
+ * scheduling matter of this kernel).  A launch runs 32 workgroups per XCD at a time, each 256 query rows of one head,
+ * and takes ceil(n_heads / 8 * ceil(n_tokens / 256) / 32) rounds however few workgroups the last one holds.  Given
+ * `split_scratch` of at least this many bytes, cdm_attn_fwd_packed_bf16 cuts the query blocks of that last round into
+ * 2, 4 or 8 units by key range and merges their results with a second, small kernel (same operator; the output
+ * differs from the single-pass one by the rounding of the partial results to bf16).  0 = nothing to split for this
+ * shape (fewer than two whole rounds, heads not a multiple of 8, a whole number of rounds, or no split that ends in
+ * half a round or less - a round with idle CUs runs faster on this power-limited chip, so less does not pay); a launch whose causal
+ * prefix reaches into the last round's query blocks is never split.  n_heads counts query heads.
+ * cdm_attn_fwd_bf16 uses what its workspace holds beyond cdm_attn_workspace_bytes (rounded up to 256) for this.
+ */
+int64_t cdm_attn_split_scratch_bytes(int64_t n_tokens, int32_t n_heads, int32_t head_dim);
 
 /*
  * cdm_attn_fwd_bf16 for callers that cannot allocate device memory or carry a workspace (code under HIP graph

@@ -103,9 +103,9 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
     assert lib.cdm_attn_fwd_bf16(*args, None, 17, None) == _lib.ERR_BAD_ARG                  # causal prefix > n_tokens
     pk = (fake, 64, None, None, fake, fake, 64, 16, 1, 1, 64, None)
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, -64, 0, None, None) == _lib.ERR_BAD_SHAPE       # negative prefix length
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 64, 0, None, None) == _lib.ERR_BAD_ARG          # prefix size without images
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 64, 4, None, None) == _lib.ERR_UNSUPPORTED      # prefix images + causal prefix
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, -64, 0, None, None, 0, None) == _lib.ERR_BAD_SHAPE       # negative prefix length
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 64, 0, None, None, 0, None) == _lib.ERR_BAD_ARG          # prefix size without images
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, fake, 64, 4, None, None, 0, None) == _lib.ERR_UNSUPPORTED      # prefix images + causal prefix
     qn = _lib.QkNorm(fake, fake, ends, 2, 0.0)
     assert lib.cdm_attn_fwd_bf16(*args, C.addressof(qn), 0, None) == _lib.ERR_BAD_ARG
     # grouped-query attention: the K/V head count must divide the query head count
@@ -114,8 +114,16 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert gq(6, 4) == _lib.ERR_BAD_SHAPE and "divide" in _lib.last_error()
     assert gq(6, 0) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_attn_fwd_packed_bf16(fake, 384, None, None, fake, fake, 384, 16, 6, 4, 64, None, None, 0, 0, None,
-                                        None) == _lib.ERR_BAD_SHAPE
-    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 0, 0, fake + 2, None) == _lib.ERR_BAD_ALIGN       # misaligned row_amax
+                                        None, 0, None) == _lib.ERR_BAD_SHAPE
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 0, 0, None, fake + 4, 1 << 20, None) == _lib.ERR_BAD_ARG   # misaligned split scratch
+    # the split of the last round: nothing below two whole rounds of workgroups per XCD, nothing on a whole number of rounds
+    assert lib.cdm_attn_split_scratch_bytes(4096, 16, 128) == 0
+    assert lib.cdm_attn_split_scratch_bytes(57344, 32, 128) == 0
+    assert lib.cdm_attn_split_scratch_bytes(56320, 32, 128) == 8 * 16 * 2 * 256 * (256 + 4)      # 16 query blocks x 2 ranges per XCD
+    assert lib.cdm_attn_split_scratch_bytes(56832, 32, 128) == 0      # 24 blocks left: no plan ends in half a round or less
+    assert lib.cdm_attn_split_scratch_bytes(29440, 32, 128) == 8 * 12 * 8 * 256 * (256 + 4)
+    assert lib.cdm_attn_split_scratch_bytes(56832, 30, 128) == 0
+    assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 0, 0, fake + 2, None, 0, None) == _lib.ERR_BAD_ALIGN       # misaligned row_amax
     # partial row maxima: only the SwiGLU epilogue of the e4m3 GEMM writes them; the quantiser that reads them checks its table
     f8 = lambda epi, amax, ld: lib.cdm_gemm_fp8(fake, 256, fake, fake, 256, fake, fake, fake, fake, 256, 8, 256, 256, epi, None, 0,
                                                 None, None, None, 0, 0, amax, ld, None)

@@ -469,6 +469,74 @@ def test_attention_with_prefix_key_images(P, m, H, hd):
     assert_close(o, want.reshape(m, d), 0.9999, 1e-2, f"prefix images P={P} m={m}")
 
 
+@pytest.mark.parametrize("n,H,Hkv,hd,P,causal,split", [(9372, 16, 16, 128, 0, 0, 8), (9372, 16, 4, 128, 100, 0, 8),
+                                                       (9500, 16, 16, 64, 0, 0, 8), (9372, 16, 16, 128, 0, 300, 8),
+                                                       (10240, 16, 8, 128, 64, 0, 2), (9372, 16, 16, 128, 0, 7000, 1)])
+def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split):
+    """A launch runs 32 workgroups (256 query rows of one head each) per XCD at a time; given scratch memory, the query
+    blocks of the last, partial round are cut into 2 / 4 / 8 units by key range and merged by a second kernel.  Checked:
+    the scratch size states the plan (2 heads per XCD x 37 query blocks = 74 = 2 x 32 + 10: ten blocks in eight ranges
+    fill 80 / 32 -> 3 eighths of a round; 2 x 40 = 80 = 2 x 32 + 16: sixteen blocks in two ranges fill one half), rows outside the
+    tail are bit-equal to the one-pass launch, rows inside differ from it by the extra rounding of the partial results
+    only, agree with the oracle, carry exact row maxima, and the launch is bit-reproducible.  With ragged prefix key
+    images, grouped K / V heads, QK-norm and mRoPE; a causal prefix short of the tail's query blocks leaves the plan
+    alone, one that reaches into them switches it off."""
+    g = gen(n + H + P)
+    d, dkv, nt = H * hd, Hkv * hd, P + n
+    pos, _ = rotary.build_positions(nt, (0, 0, 0), 0)
+    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48) if hd == 128 else (16, 24, 24))
+    cosd, sind = cos.to(dev()), sin.to(dev())
+    qkv, qkvr = rand_bf16((nt, d + 2 * dkv), g, 1.5)
+    qw, kw = 1 + 0.2 * torch.randn(1, hd, generator=g), 1 + 0.2 * torch.randn(1, hd, generator=g)
+    qwd, kwd = qw.to(dev()), kw.to(dev())
+    q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
+    qk = lambda m: (qwd, kwd, [m], 1e-6)
+    pre = None
+    if P:
+        pre = (ops.attention_pack_kv(k[:P], v[:P], Hkv, hd, cos=cosd[:P].contiguous(), sin=sind[:P].contiguous(), qk_norm=qk(P)), P)
+    rot = dict(cos=cosd[P:].contiguous(), sin=sind[P:].contiguous())
+    img = ops.attention_pack_kv(k[P:], v[P:], Hkv, hd, qk_norm=qk(n), **rot)
+    nqb, per_xcd = (n + 255) // 256, (H // 8) * ((n + 255) // 256)
+    tail = per_xcd % 32
+    cost = {s_: -(-tail * s_ // 32) / s_ for s_ in (2, 4, 8)}
+    planned = min(cost, key=lambda s_: (cost[s_], s_))
+    assert planned == (split if split > 1 else 8) and tail > 0
+    want_bytes = 8 * tail * planned * 256 * (2 * hd + 4)
+    assert ops.attn_split_scratch_bytes(n, H, hd) == want_bytes
+    scratch = torch.empty((want_bytes,), dtype=torch.uint8, device=dev())
+    kw_args = dict(qk_norm=qk(n), prefix=pre, causal_prefix=causal, n_kv_heads=Hkv, **rot)
+    amax = torch.full((n, H), float("nan"), dtype=torch.float32, device=dev())
+    one = ops.attention_packed(q[P:], img, H, hd, **kw_args)                        # the images alone: one pass
+    two = ops.attention_packed(q[P:], img, H, hd, split_scratch=scratch, row_amax=amax, **kw_args)
+    assert torch.equal(two, ops.attention_packed(q[P:], img, H, hd, split_scratch=scratch, **kw_args))
+    assert torch.equal(amax, two.float().abs().view(n, H, hd).amax(-1))
+    # the tail: the last `tail` (head, query block) pairs of every XCD, heads dealt H / 8 per XCD, query blocks fastest
+    in_tail = torch.zeros(n, H, dtype=torch.bool)
+    for x in range(8):
+        for kk in range(per_xcd - tail, per_xcd):
+            in_tail[(kk % nqb) * 256:(kk % nqb + 1) * 256, x * (H // 8) + kk // nqb] = True
+    m3 = in_tail.to(dev())[:, :, None].expand(n, H, hd).reshape(n, d)
+    if split == 1:
+        assert torch.equal(one, two)
+        return
+    assert torch.equal(one[~m3], two[~m3])
+    assert not torch.equal(one[m3], two[m3])
+    assert_close(two[m3], one[m3].float().cpu(), 0.99999, 8e-3, f"split vs one pass n={n} H={H}/{Hkv} hd={hd} P={P} causal={causal}")
+    # oracle on sampled rows of the tail, two heads
+    rows = torch.unique(torch.cat([torch.arange(n - 40, n), torch.randint((per_xcd - tail) % nqb * 256, n, (88,), generator=g)]))
+    grp = H // Hkv
+    for h in (H // 8 - 1, H - 1):
+        assert bool(in_tail[rows, h].all())
+        hk = h // grp
+        qn = O.apply_mrope(O.rms_norm(qkvr[P:, :d].view(n, H, hd)[rows][:, h:h + 1], qw[0], 1e-6), cos[P:][rows], sin[P:][rows])
+        kn = O.apply_mrope(O.rms_norm(qkvr[:, d:d + dkv].view(nt, Hkv, hd)[:, hk:hk + 1], kw[0], 1e-6), cos, sin)
+        vv = qkvr[:, d + dkv:].view(nt, Hkv, hd)[:, hk:hk + 1]
+        if causal:      # sampled rows lie behind the causal prefix: they see every key
+            assert int(rows.min()) >= causal
+        want = O.attention(qn, kn, vv)
+        assert_close(two.view(n, H, hd)[rows.to(dev()), h], want[:, 0], 0.9999, 1e-2, f"split vs oracle head {h}")
+
+
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("n,hd", [(100, 64), (200, 128), (70, 128), (64, 64)])
 def test_attention_with_strongly_negative_logits(n, hd, variant, request):
