@@ -515,10 +515,11 @@ def test_c2_full_size_cached_context_forward():
     upd = xj[rows]
     assert float((want - upd).abs().max()) > 0.5
     assert_close(got.float().cpu() - upd, want - upd, 0.999, BF16_REL, "C2 cached-context forward: the update alone")
-    # the joint forward under the same mask gives the same video rows (K of the text run is rounded once more there
-    # or here depending on the path, hence a tolerance instead of equality)
+    # the joint forward under the same mask gives the same video rows; a tolerance instead of equality: 220 query blocks
+    # per head end in half a round of workgroups, which the cached forward splits by key range (its partial results are
+    # rounded to bf16 once more), while the joint forward's 222 are left alone
     joint = st(xv, t, encoder_hidden_states=xt, return_dict=True)["joint"]
-    assert_close(first, joint[P:].float().cpu(), 0.99999, 4e-3, "cached context == joint forward at full size")
+    assert_close(first, joint[P:].float().cpu(), 0.99999, 8e-3, "cached context == joint forward at full size")
     again = st(xv, t, return_dict=True, context_cache=cache)["joint"]
     assert torch.equal(first, again), "cached-context forward differs between identical launches"
 
