@@ -222,7 +222,9 @@ def bench_attention_only(cfg, steps, warmup, dev, attn_variant=0):
     pos, _ = rotary.build_positions(0, cfg.grid, 0)
     cos, sin = rotary.rotary_tables(pos, hd, cfg.mrope_sections, cfg.rope_base, cfg.rope_layout, dev)
     out = torch.empty((n, d), dtype=torch.bfloat16, device=dev)
-    ws = torch.empty(ops.attn_workspace_bytes(n, H, hd), dtype=torch.uint8, device=dev)
+    # K / V tile images plus the scratch of the split of the last round of workgroups (220 query blocks x 4 heads per XCD
+    # = 27.5 rounds of 32: the last 16 blocks of every XCD run as two key ranges each)
+    ws = torch.empty(ops.attn_workspace_total_bytes(n, H, H, hd), dtype=torch.uint8, device=dev)
     step = lambda: ops.attention(qkv[:, :d], qkv[:, d:2 * d], qkv[:, 2 * d:], H, hd, out=out, workspace=ws, cos=cos, sin=sin)
     ms, ev, _, _ = time_steps(step, steps, warmup)
     assert bool(torch.isfinite(out.float()).all()), "non-finite output"
