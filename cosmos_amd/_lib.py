@@ -59,6 +59,7 @@ SIGNATURES = {
     "cdm_attn_fwd_packed_bf16": (_I32, [_P, _I64, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _P, _I64, _I64, _P, _P,
                                         _I64, _P]),
     "cdm_attn_split_scratch_bytes": (_I64, [_I64, _I32, _I32]),
+    "cdm_linear_bias_bf16": (_I32, [_P, _I64, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "cdm_grouped_gemm_fp8": (_I32, [_P, _I64, _P, C.POINTER(_P), C.POINTER(_P), _I64, C.POINTER(_P), C.POINTER(_P), _P, _I64,
                                     C.POINTER(_I64), C.POINTER(_I64), _I32, _I64, _I64, _I32, _P, _I64, C.POINTER(_P), _P,
                                     _P, _I64, _I32, _P, _I64, _P]),

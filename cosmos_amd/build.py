@@ -21,7 +21,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcosmos_dm_hip.so")
 CROSSCHECK_PATH = os.path.join(LIB_DIR, "libcosmos_dm_hip_crosscheck.so")
-SOURCES = ["api.hip", "norm.hip", "rope.hip", "gemm.hip", "attn.hip", "step.hip"]
+SOURCES = ["api.hip", "norm.hip", "rope.hip", "gemm.hip", "attn.hip", "step.hip", "edge.hip"]
 # packed fp32 VALU forms are switched off on purpose (hipcc's host pass warns that it does not
 # know the feature; that warning is harmless)
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",

@@ -739,6 +739,12 @@ class GraphedStack:
         return self.out
 
 
+def _edge_linear(lin: nn.Linear, x: torch.Tensor) -> torch.Tensor:
+    """A narrow linear layer with bias at the edge of the stack (patchify / un-patchify, action and audio
+    projections) through the HIP kernel made for it; ``lin`` only holds the parameters under their checkpoint names."""
+    return ops.linear_bias(x if x.stride(-1) == 1 else x.contiguous(), lin.weight, lin.bias)
+
+
 class DMTransformer(nn.Module):
     """The transformer-shaped object a diffusers pipeline drives (``pipe.transformer``): latents in, velocity out.
 
@@ -838,13 +844,13 @@ class DMTransformer(nn.Module):
                                                       _sample(audio_states, b, 3, batch)),
                                batch, return_dict)
         dt = self.proj_in.weight.dtype
-        tok = self.proj_in(self.patchify(hidden_states[0].to(dt)))
+        tok = _edge_linear(self.proj_in, self.patchify(hidden_states[0].to(dt)))
         given = {"audio": audio_states, "action": action_states}
         emb = {}
         for name, _, p_in, _, embed in self._streams():
             if given[name] is None:
                 raise ValueError(f"this configuration expects {name}_states")
-            emb[name] = p_in(_as2d(given[name]).to(dt)) + embed
+            emb[name] = _edge_linear(p_in, _as2d(given[name]).to(dt)) + embed
         res = self.stack(tok, timestep, encoder_hidden_states=None if context_cache is not None else encoder_hidden_states,
                          action_states=emb.get("action"), return_dict=True, context_cache=context_cache,
                          audio_states=emb.get("audio"))
@@ -852,10 +858,10 @@ class DMTransformer(nn.Module):
         first = 0 if context_cache is not None else c.n_text
         y = ops.adaln_rmsnorm(joint, self.norm_out.data, None, None, c.eps)
         video = y[first:first + c.n_video]
-        sample = self.unpatchify(self.proj_out(video))
+        sample = self.unpatchify(_edge_linear(self.proj_out, video))
         outs, at = {"audio": None, "action": None}, first + c.n_video
         for name, n, _, p_out, _ in self._streams():
-            outs[name] = p_out(y[at:at + n]).unsqueeze(0)
+            outs[name] = _edge_linear(p_out, y[at:at + n]).unsqueeze(0)
             at += n
         if return_dict:
             return {"sample": sample, **outs}

@@ -212,6 +212,28 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
     return out
 
 
+@_timed("edge")
+def linear_bias(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T + bias[N] for the narrow linear layers at the edges of the stack (patchify /
+    un-patchify, action and audio projections); bf16 in / fp32 accumulate / bf16 out; any widths (16-byte accesses where
+    rows are 16-byte aligned and N, K are multiples of 8)."""
+    lib = _lib.load()
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or (bias is not None and bias.shape != (N,)):
+        raise ValueError("weight / bias shape mismatch")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    if out.shape != (M, N):
+        raise ValueError("out shape mismatch")
+    rc = lib.cdm_linear_bias_bf16(_chk(a, "a", torch.bfloat16, 2), a.stride(0), _chk(w, "w", torch.bfloat16, 2), w.stride(0),
+                                  _chk(bias, "bias", torch.bfloat16, 1), _chk(out, "out", torch.bfloat16, 2), out.stride(0),
+                                  M, N, K, _stream())
+    _lib.check(rc, "cdm_linear_bias_bf16")
+    return out
+
+
 @_timed("gemm")
 def gemm_fp8(aq: torch.Tensor, sa: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, *,
              w2q: Optional[torch.Tensor] = None, sw2: Optional[torch.Tensor] = None, epilogue: str = "none",

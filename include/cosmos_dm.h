@@ -261,6 +261,19 @@ int32_t cdm_attn_fwd_static_bf16(const void* q, int64_t ldq, const void* k, int6
                                  int64_t causal_prefix, void* stream);
 
 /*
+ * Linear layer WITH bias at the edges of the stack - replaces nn.Linear of proj_in / proj_out (patchify and
+ * un-patchify projections), action_proj_in / action_proj_out and audio_proj_in / audio_proj_out (parameter names:
+ * transformers models/cosmos3_omni/modeling_cosmos3_omni.py:48-58), where K or N is a few dozen elements and the
+ * layer is bound by moving the token rows once.
+ *   A: [M, K] (lda), W: [N, K] (ldw) row-major like nn.Linear.weight, bias: [N] bf16 or null, C: [M, N] (ldc), all bf16;
+ *   fp32 accumulation on MFMA, bias added in fp32, one rounding to bf16.
+ * Any M, N, K >= 1 (a last partial 32-wide k-step is zero-filled).  16-byte accesses are used where A, W, C and their row
+ * strides are 16-byte aligned and N, K are multiples of 8; other shapes (an action stream 6 wide) go element by element.
+ */
+int32_t cdm_linear_bias_bf16(const void* A, int64_t lda, const void* W, int64_t ldw, const void* bias, void* C,
+                             int64_t ldc, int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
  * Mixture-of-Transformers routed linear: contiguous token segments, one weight set each
  * (README.md:53,74 - per-modality weights around one shared attention).  Equivalent to
  * cdm_gemm_bf16 on rows [seg_start[g], seg_start[g] + seg_len[g]) with W[g] (and W2[g], gate[g]).

@@ -124,6 +124,10 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_attn_split_scratch_bytes(29440, 32, 128) == 8 * 12 * 8 * 256 * (256 + 4)
     assert lib.cdm_attn_split_scratch_bytes(56832, 30, 128) == 0
     assert lib.cdm_attn_fwd_packed_bf16(*pk, None, 0, 0, fake + 2, None, 0, None) == _lib.ERR_BAD_ALIGN       # misaligned row_amax
+    # edge linear: strides must cover the rows
+    assert lib.cdm_linear_bias_bf16(fake, 8, fake, 64, None, fake, 64, 4, 64, 64, None) == _lib.ERR_BAD_ARG
+    assert lib.cdm_linear_bias_bf16(fake, 64, fake, 64, fake + 1, fake, 64, 4, 64, 64, None) == _lib.ERR_BAD_ALIGN
+    assert lib.cdm_linear_bias_bf16(fake, 64, fake, 64, None, fake, 64, 0, 64, 64, None) == _lib.OK          # no rows: nothing to launch
     # partial row maxima: only the SwiGLU epilogue of the e4m3 GEMM writes them; the quantiser that reads them checks its table
     f8 = lambda epi, amax, ld: lib.cdm_gemm_fp8(fake, 256, fake, fake, 256, fake, fake, fake, fake, 256, 8, 256, 256, epi, None, 0,
                                                 None, None, None, 0, 0, amax, ld, None)

@@ -168,6 +168,28 @@ def test_gemm_rope_qk(hd, H, sections, variant, request):
     assert_close(c[:, 2 * d:], want[:, 2 * d:], 0.99999, 6e-3, "rope_qk v")
 
 
+@pytest.mark.parametrize("M,N,K,bias", [(1000, 4096, 64, True), (1000, 64, 4096, True), (300, 16, 512, False), (77, 6, 256, True),
+                                        (256, 512, 6, True), (5, 10, 40, True), (64, 264, 16, True), (1, 8, 8, False)])
+def test_linear_bias_at_the_stack_edges(M, N, K, bias):
+    """The narrow linear layers with bias (patchify / un-patchify, action and audio projections): x W^T + b against fp32,
+    one rounding to bf16.  Widths that are no multiple of 8 take the element-wise path; row-strided views of the
+    operands and of the output are honoured and nothing beyond the output's columns is written."""
+    g = gen(M + N + K)
+    x, xr = rand_bf16((M, K + 8), g)
+    w, wr = rand_bf16((N, K), g, 0.1)
+    b, br = rand_bf16((N,), g) if bias else (None, None)
+    out = torch.full((M, N + 3), 7.0, dtype=torch.bfloat16, device=dev())
+    got = ops.linear_bias(x[:, :K], w, b, out=out[:, :N])
+    want = xr[:, :K] @ wr.t() + (br if bias else 0.0)
+    assert_close(got, want, 0.99999, 4e-3, f"edge linear {M}x{N}x{K}")
+    assert bool((out[:, N:] == 7.0).all())
+    # contiguous operands and output (16-byte accesses where the widths allow; the k-steps are then summed in another
+    # order): the same values up to the last bit of the rounding, and bit-equal from call to call
+    again = ops.linear_bias(x[:, :K].contiguous(), w, b)
+    assert float((got.float() - again.float()).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
+    assert torch.equal(again, ops.linear_bias(x[:, :K].contiguous(), w, b))
+
+
 def test_grouped_gemm_three_segments():
     g = gen(77)
     K, N = 256, 264
