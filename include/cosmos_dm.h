@@ -247,6 +247,8 @@ int64_t cdm_attn_split_scratch_bytes(int64_t n_tokens, int32_t n_heads, int32_t 
  * operator and all other arguments are those of cdm_attn_fwd_bf16.  The K / V tile images go into a device array
  * built into the library (CDM_ATTN_STATIC_SCRATCH_BYTES per GPU, held until the process ends); the call allocates
  * nothing.  Shapes whose images (cdm_attn_workspace_bytes) exceed that size are rejected with CDM_ERR_BAD_SHAPE.
+ * The result is bit-equal to cdm_attn_fwd_bf16 with a workspace of exactly cdm_attn_workspace_bytes (the array holds
+ * no scratch for a split of the last round of workgroups).
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
  * threads) race; calls on one stream are ordered and need no clearing in between (every call rewrites all
  * tiles it reads, padding included).  The array's address is looked up once per device, by the first call on that
