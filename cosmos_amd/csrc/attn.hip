@@ -478,8 +478,10 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
     }
 
     // key tiles: NP whole tiles of the prefix images, then the NM tiles of the main images
-    // keys of the frame: a range that ends ahead of the sequence's last tile ends on a full tile
-    const int n_keys = t1 < NT_all ? NT * BN : p.n_prefix_tiles * BN + p.n_tokens - t0 * BN;
+    // keys of the frame: a range that ends ahead of the sequence's last tile ends on a full tile - unless that tile is the
+    // prefix's partly filled last one, which then is this frame's ragged last tile (prefix_last_valid = BN otherwise)
+    const int n_keys = t1 < NT_all ? NT * BN - (t1 == p.n_prefix_tiles ? BN - p.prefix_last_valid : 0)
+                                   : p.n_prefix_tiles * BN + p.n_tokens - t0 * BN;
     const int last_valid = n_keys - (NT - 1) * BN;
     // per-row key limit and the tiles this workgroup needs: a query block inside the causal prefix stops at its
     // own last row, and every tile it visits is masked per row
@@ -641,7 +643,10 @@ __global__ __launch_bounds__(512 / QS) __attribute__((amdgpu_waves_per_eu(2 / QS
             amax = fmaxf(fmaxf(amax, fmaxf(fabsf(bf16lo(w.x)), fabsf(bf16hi(w.x)))), fmaxf(fabsf(bf16lo(w.y)), fabsf(bf16hi(w.y))));
         }
         if (unit >= 0) {      // a split unit leaves log2 of its sum of exponentials (reference added back) beside its rows
-            if (g4 == 0) p.part_lse[(int64_t)unit * BMQ + wave * (32 * QS) + qb * 16 + r16] = __log2f(l_tot) - negm[qb][0];
+            // (a LATE kernel keeps the reference in the units of its accumulators: late_r times that is the exponent's)
+            if (g4 == 0)
+                p.part_lse[(int64_t)unit * BMQ + wave * (32 * QS) + qb * 16 + r16] =
+                    __log2f(l_tot) - negm[qb][0] * (LATE ? p.late_r : 1.0f);
         } else if (p.row_amax != nullptr) {      // the row's channels of this head are spread over the four quarter-waves
             amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
             amax = fmaxf(amax, __shfl_xor(amax, 32, 64));

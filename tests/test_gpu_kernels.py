@@ -491,10 +491,11 @@ def test_attention_with_prefix_key_images(P, m, H, hd):
     assert_close(o, want.reshape(m, d), 0.9999, 1e-2, f"prefix images P={P} m={m}")
 
 
+@pytest.mark.parametrize("plain", [False, True])
 @pytest.mark.parametrize("n,H,Hkv,hd,P,causal,split", [(9372, 16, 16, 128, 0, 0, 8), (9372, 16, 4, 128, 100, 0, 8),
                                                        (9500, 16, 16, 64, 0, 0, 8), (9372, 16, 16, 128, 0, 300, 8),
                                                        (10240, 16, 8, 128, 64, 0, 2), (9372, 16, 16, 128, 0, 7000, 1)])
-def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split):
+def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split, plain):
     """A launch runs 32 workgroups (256 query rows of one head each) per XCD at a time; given scratch memory, the query
     blocks of the last, partial round are cut into 2 / 4 / 8 units by key range and merged by a second kernel.  Checked:
     the scratch size states the plan (2 heads per XCD x 37 query blocks = 74 = 2 x 32 + 10: ten blocks in eight ranges
@@ -502,7 +503,10 @@ def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split):
     tail are bit-equal to the one-pass launch, rows inside differ from it by the extra rounding of the partial results
     only, agree with the oracle, carry exact row maxima, and the launch is bit-reproducible.  With ragged prefix key
     images, grouped K / V heads, QK-norm and mRoPE; a causal prefix short of the tail's query blocks leaves the plan
-    alone, one that reaches into them switches it off."""
+    alone, one that reaches into them switches it off.  ``plain``: neither QK-norm nor rotation - the kernel form that
+    applies part of the softmax scale to the fp32 scores, whose reference lives in other units."""
+    if plain and (causal or split == 1):
+        pytest.skip("the plain form is covered by the other cases")
     g = gen(n + H + P)
     d, dkv, nt = H * hd, Hkv * hd, P + n
     pos, _ = rotary.build_positions(nt, (0, 0, 0), 0)
@@ -512,11 +516,12 @@ def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split):
     qw, kw = 1 + 0.2 * torch.randn(1, hd, generator=g), 1 + 0.2 * torch.randn(1, hd, generator=g)
     qwd, kwd = qw.to(dev()), kw.to(dev())
     q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
-    qk = lambda m: (qwd, kwd, [m], 1e-6)
+    qk = lambda m: None if plain else (qwd, kwd, [m], 1e-6)
     pre = None
     if P:
-        pre = (ops.attention_pack_kv(k[:P], v[:P], Hkv, hd, cos=cosd[:P].contiguous(), sin=sind[:P].contiguous(), qk_norm=qk(P)), P)
-    rot = dict(cos=cosd[P:].contiguous(), sin=sind[P:].contiguous())
+        pre_rot = {} if plain else dict(cos=cosd[:P].contiguous(), sin=sind[:P].contiguous())
+        pre = (ops.attention_pack_kv(k[:P], v[:P], Hkv, hd, qk_norm=qk(P), **pre_rot), P)
+    rot = {} if plain else dict(cos=cosd[P:].contiguous(), sin=sind[P:].contiguous())
     img = ops.attention_pack_kv(k[P:], v[P:], Hkv, hd, qk_norm=qk(n), **rot)
     nqb, per_xcd = (n + 255) // 256, (H // 8) * ((n + 255) // 256)
     tail = per_xcd % 32
@@ -543,15 +548,17 @@ def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split):
         return
     assert torch.equal(one[~m3], two[~m3])
     assert not torch.equal(one[m3], two[m3])
-    assert_close(two[m3], one[m3].float().cpu(), 0.99999, 8e-3, f"split vs one pass n={n} H={H}/{Hkv} hd={hd} P={P} causal={causal}")
+    assert_close(two[m3], one[m3].float().cpu(), 0.99999, 8e-3, f"split vs one pass n={n} H={H}/{Hkv} hd={hd} P={P} causal={causal} plain={plain}")
     # oracle on sampled rows of the tail, two heads
     rows = torch.unique(torch.cat([torch.arange(n - 40, n), torch.randint((per_xcd - tail) % nqb * 256, n, (88,), generator=g)]))
     grp = H // Hkv
     for h in (H // 8 - 1, H - 1):
         assert bool(in_tail[rows, h].all())
         hk = h // grp
-        qn = O.apply_mrope(O.rms_norm(qkvr[P:, :d].view(n, H, hd)[rows][:, h:h + 1], qw[0], 1e-6), cos[P:][rows], sin[P:][rows])
-        kn = O.apply_mrope(O.rms_norm(qkvr[:, d:d + dkv].view(nt, Hkv, hd)[:, hk:hk + 1], kw[0], 1e-6), cos, sin)
+        qn, kn = qkvr[P:, :d].view(n, H, hd)[rows][:, h:h + 1], qkvr[:, d:d + dkv].view(nt, Hkv, hd)[:, hk:hk + 1]
+        if not plain:
+            qn = O.apply_mrope(O.rms_norm(qn, qw[0], 1e-6), cos[P:][rows], sin[P:][rows])
+            kn = O.apply_mrope(O.rms_norm(kn, kw[0], 1e-6), cos, sin)
         vv = qkvr[:, d + dkv:].view(nt, Hkv, hd)[:, hk:hk + 1]
         if causal:      # sampled rows lie behind the causal prefix: they see every key
             assert int(rows.min()) >= causal
@@ -576,6 +583,36 @@ def test_attention_with_strongly_negative_logits(n, hd, variant, request):
     want = O.attention(qr.float().view(n, 1, hd), kr.float().view(n, 1, hd), vr.float().view(n, 1, hd)).reshape(n, hd)
     assert float((qr.float() @ kr.float().t()).max()) / math.sqrt(hd) < -100.0
     assert_close(o, want, 0.9999, 1e-2, f"attention with strongly negative logits n={n}")
+
+
+@pytest.mark.parametrize("variant", [0, 2])
+def test_split_range_that_ends_on_the_ragged_prefix_tile(variant, request):
+    """64 heads x 10 query blocks = 80 workgroups per XCD: the last 16 run as two key ranges each, and with 40 prefix
+    tiles ahead of 40 main tiles the first range ends exactly on the prefix's last tile, of which 4 keys exist.  Every
+    score is far below zero, so a zero key of that tile's padding - in the step that masks it, or in the surplus step
+    behind the range's end, which looks at the same tile again - would be the row maximum and scale the sums towards zero
+    wherever row maxima are taken (variant 2: everywhere)."""
+    prev = ops.set_variant("attn", variant)
+    request.addfinalizer(lambda: ops.set_variant("attn", prev))
+    P, n, H, hd = 39 * 64 + 4, 2560, 64, 64
+    g = gen(77)
+    c = (120.0 * math.sqrt(hd) / hd) ** 0.5
+    kr = (c + 0.05 * torch.randn(P + n, hd, generator=g)).to(torch.bfloat16)
+    qr = (-c + 0.05 * torch.randn(n, hd, generator=g)).to(torch.bfloat16)
+    vr = torch.randn(P + n, hd, generator=g).to(torch.bfloat16)
+    rep = lambda t: t.to(dev()).unsqueeze(1).expand(t.shape[0], H, hd).reshape(t.shape[0], H * hd).contiguous()
+    q, k, v = rep(qr), rep(kr), rep(vr)
+    assert ops.attn_split_scratch_bytes(n, H, hd) == 8 * 16 * 2 * 256 * (2 * hd + 4)
+    pre = (ops.attention_pack_kv(k[:P], v[:P], H, hd), P)
+    img = ops.attention_pack_kv(k[P:], v[P:], H, hd)
+    scratch = torch.empty((ops.attn_split_scratch_bytes(n, H, hd),), dtype=torch.uint8, device=dev())
+    one = ops.attention_packed(q, img, H, hd, prefix=pre)
+    two = ops.attention_packed(q, img, H, hd, prefix=pre, split_scratch=scratch)
+    assert not torch.equal(one, two)                                  # the split ran
+    want = O.attention(qr.float().view(n, 1, hd), kr.float().view(P + n, 1, hd), vr.float().view(P + n, 1, hd)).reshape(n, hd)
+    for h in (0, 7, 63):      # head 7: the last of XCD 0, whose query blocks 2 .. 9 and those of head 6 are split; 0: not split
+        assert_close(two.view(n, H, hd)[:, h], want, 0.9999, 1e-2, f"split range ending on the ragged prefix tile, head {h}")
+        assert_close(one.view(n, H, hd)[:, h], want, 0.9999, 1e-2, f"one pass, head {h}")
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2])
