@@ -515,6 +515,10 @@ def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split, plain):
     qkv, qkvr = rand_bf16((nt, d + 2 * dkv), g, 1.5)
     qw, kw = 1 + 0.2 * torch.randn(1, hd, generator=g), 1 + 0.2 * torch.randn(1, hd, generator=g)
     qwd, kwd = qw.to(dev()), kw.to(dev())
+    if plain:      # two outlier keys (nothing normalises them here): their tiles take the row maxima, inside split ranges too
+        for key, f in ((P + 77, 10.0), (P + 5000, 12.0)):
+            qkvr[key, d:d + dkv] = (qkvr[key, d:d + dkv] * f).to(torch.bfloat16).float()
+        qkv = qkvr.to(torch.bfloat16).to(dev())
     q, k, v = qkv[:, :d], qkv[:, d:d + dkv], qkv[:, d + dkv:]
     qk = lambda m: None if plain else (qwd, kwd, [m], 1e-6)
     pre = None
