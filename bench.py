@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a plain streaming
 # kernel of known size (FETCH_SIZE unit = 2 KiB, WRITE_SIZE unit = 1 KiB on this chip).  Counters cannot be read
 # from inside this process; the figure is only reported while the kernel's source is the one it was measured on.
-ATTN_TRAFFIC = {"shape": (56832, 32, 128), "bytes": 8.616e9 + 0.466e9, "attn_source_sha256_16": "fd739a7a1bc49c10"}
+ATTN_TRAFFIC = {"shape": (56832, 32, 128), "bytes": 8.616e9 + 0.466e9, "attn_source_sha256_16": "e241ef1061e23461"}
 
 T_START = time.perf_counter()
 
