@@ -751,8 +751,9 @@ class DMTransformer(nn.Module):
     Stack edges around ``DMStack``: patchify + ``proj_in``, the block stack, a final RMSNorm, ``proj_out`` +
     unpatchify; an optional action stream (``action_proj_in`` + ``action_modality_embed`` in, ``action_proj_out``
     out) and an optional audio stream (``audio_proj_in`` + ``audio_modality_embed`` in, ``audio_proj_out`` out: the
-    sound the reference generates with ``enable_sound``, README.md:259).  The edge linears are one-off projections with K or N = patch width (64 for 16 latent channels and 1x2x2
-    patches): 0.1 % of a step's flops, they stay on the stock BLAS path like the one-row timestep MLP.  Parameter
+    sound the reference generates with ``enable_sound``, README.md:259).  The edge linears are one-off projections with
+    K or N = patch width (64 for 16 latent channels and 1x2x2 patches), bound by moving the token rows once: they run
+    through ``ops.linear_bias``; the ``nn.Linear`` modules only hold the parameters.  Parameter
     names follow the checkpoint keys the reference's model files attest (``proj_in``, ``proj_out``,
     ``time_embedder``, ``action_proj_in``, ``action_proj_out``, ``action_modality_embed``, ``audio_proj_in``,
     ``audio_proj_out``, ``audio_modality_embed``); the patch order
