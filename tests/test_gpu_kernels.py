@@ -491,10 +491,13 @@ def test_attention_with_prefix_key_images(P, m, H, hd):
     assert_close(o, want.reshape(m, d), 0.9999, 1e-2, f"prefix images P={P} m={m}")
 
 
-@pytest.mark.parametrize("plain", [False, True])
-@pytest.mark.parametrize("n,H,Hkv,hd,P,causal,split", [(9372, 16, 16, 128, 0, 0, 8), (9372, 16, 4, 128, 100, 0, 8),
-                                                       (9500, 16, 16, 64, 0, 0, 8), (9372, 16, 16, 128, 0, 300, 8),
-                                                       (10240, 16, 8, 128, 64, 0, 2), (9372, 16, 16, 128, 0, 7000, 1)])
+_SPLIT_SHAPES = [(9372, 16, 16, 128, 0, 0, 8), (9372, 16, 4, 128, 100, 0, 8), (9500, 16, 16, 64, 0, 0, 8),
+                 (10240, 16, 8, 128, 64, 0, 2)]
+
+
+@pytest.mark.parametrize("n,H,Hkv,hd,P,causal,split,plain",
+                         [c + (False,) for c in _SPLIT_SHAPES] + [c + (True,) for c in _SPLIT_SHAPES]
+                         + [(9372, 16, 16, 128, 0, 300, 8, False), (9372, 16, 16, 128, 0, 7000, 1, False)])
 def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split, plain):
     """A launch runs 32 workgroups (256 query rows of one head each) per XCD at a time; given scratch memory, the query
     blocks of the last, partial round are cut into 2 / 4 / 8 units by key range and merged by a second kernel.  Checked:
@@ -505,8 +508,6 @@ def test_attention_last_round_split(n, H, Hkv, hd, P, causal, split, plain):
     images, grouped K / V heads, QK-norm and mRoPE; a causal prefix short of the tail's query blocks leaves the plan
     alone, one that reaches into them switches it off.  ``plain``: neither QK-norm nor rotation - the kernel form that
     applies part of the softmax scale to the fp32 scores, whose reference lives in other units."""
-    if plain and (causal or split == 1):
-        pytest.skip("the plain form is covered by the other cases")
     g = gen(n + H + P)
     d, dkv, nt = H * hd, Hkv * hd, P + n
     pos, _ = rotary.build_positions(nt, (0, 0, 0), 0)
