@@ -169,7 +169,8 @@ def test_gemm_rope_qk(hd, H, sections, variant, request):
 
 
 @pytest.mark.parametrize("M,N,K,bias", [(1000, 4096, 64, True), (1000, 64, 4096, True), (300, 16, 512, False), (77, 6, 256, True),
-                                        (256, 512, 6, True), (5, 10, 40, True), (64, 264, 16, True), (1, 8, 8, False)])
+                                        (256, 512, 6, True), (5, 10, 40, True), (64, 264, 16, True), (1, 8, 8, False),
+                                        (200, 136, 200, True), (130, 100, 150, True), (2000, 320, 1024, False)])
 def test_linear_bias_at_the_stack_edges(M, N, K, bias):
     """The narrow linear layers with bias (patchify / un-patchify, action and audio projections): x W^T + b against fp32,
     one rounding to bf16.  Widths that are no multiple of 8 take the element-wise path; row-strided views of the
