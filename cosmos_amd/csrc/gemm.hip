@@ -326,13 +326,15 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
         }
         return;
     }
-    // QKV_PACK: 0 = Q columns (plain output), 1 = one K head, 2 = one V head (wave-uniform; head_dim is 128)
+    // QKV_PACK: 0 = Q columns (plain output), 1 = K, 2 = V (wave-uniform: the wave's 128 columns are one head of 128
+    // channels or two heads of 64, and d_q, d_kv are multiples of 128)
     const int region = EPI != CDM_EPI_QKV_PACK ? 0 : (colw < p.d_q ? 0 : (colw < p.d_q + p.d_kv ? 1 : 2));
     if (EPI == CDM_EPI_QKV_PACK && (colw >= p.N || (region != 0 && row0 >= t.m_end))) return;   // no such head / key tile
     const bool rope = (EPI == CDM_EPI_ROPE_QK && colw < p.rope_cols) ||   // wave-uniform: whole heads of Q or K
                       (EPI == CDM_EPI_QKV_PACK && region == 1 && p.cos != nullptr);
     const int half = p.head_dim >> 1;
-    float ksq = 0.0f;      // QKV_PACK, K head: largest squared norm among the lane's rows (as stored, rounded to bf16)
+    const bool hd64 = EPI == CDM_EPI_QKV_PACK && p.head_dim == 64;      // columns cs < CS/2 are one head, the others the next
+    float ksq[2] = {0.0f, 0.0f};      // QKV_PACK, K: largest squared norm among the lane's rows (as stored, rounded to bf16), per head
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
         const int rl = ACC::row_local(rs, lane), row = row0 + rl;
@@ -359,17 +361,22 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
         if (EPI == CDM_EPI_QKV_PACK && region == 1 && t.knw != nullptr) {
             // per-head RMSNorm of K on the fp32 accumulators, ahead of the rotation: the wave's 128 columns are one head,
             // a key's channels are spread over the four quarter-waves (lanes r, r + 16, r + 32, r + 48 share the row)
-            float ss = 0.0f;
+            float ss[2] = {0.0f, 0.0f};      // the two halves of the wave's columns
 #pragma unroll
             for (int cs = 0; cs < CS; ++cs)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) ss += acc.get(rs, cs, e) * acc.get(rs, cs, e);
-            ss += __shfl_xor(ss, 16, 64);
-            ss += __shfl_xor(ss, 32, 64);
-            const float rn = rsqrtf(ss * (1.0f / 128.0f) + p.k_eps);
+                for (int e = 0; e < 4; ++e) ss[cs / (CS / 2)] += acc.get(rs, cs, e) * acc.get(rs, cs, e);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                ss[h] += __shfl_xor(ss[h], 16, 64);
+                ss[h] += __shfl_xor(ss[h], 32, 64);
+            }
+            const float rn2[2] = {hd64 ? rsqrtf(ss[0] * (1.0f / 64.0f) + p.k_eps) : rsqrtf((ss[0] + ss[1]) * (1.0f / 128.0f) + p.k_eps),
+                                  hd64 ? rsqrtf(ss[1] * (1.0f / 64.0f) + p.k_eps) : rsqrtf((ss[0] + ss[1]) * (1.0f / 128.0f) + p.k_eps)};
 #pragma unroll
             for (int cs = 0; cs < CS; ++cs) {
-                const float4 w4 = *reinterpret_cast<const float4*>(t.knw + ACC::col_local(cs, lane));
+                const float rn = rn2[cs / (CS / 2)];
+                const float4 w4 = *reinterpret_cast<const float4*>(t.knw + (ACC::col_local(cs, lane) & (p.head_dim - 1)));
                 acc.set(rs, cs, 0, acc.get(rs, cs, 0) * (rn * w4.x));
                 acc.set(rs, cs, 1, acc.get(rs, cs, 1) * (rn * w4.y));
                 acc.set(rs, cs, 2, acc.get(rs, cs, 2) * (rn * w4.z));
@@ -409,7 +416,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
         }
         bf16_t* crow = p.C + (int64_t)row * p.ldc;
         const bf16_t* rrow = EPI == CDM_EPI_GATE_RESIDUAL ? p.R + (int64_t)row * p.ldr : nullptr;
-        float rsq = 0.0f;
+        float rsq[2] = {0.0f, 0.0f};
 #pragma unroll
         for (int cs = 0; cs < CS; ++cs) {
             const int cl = ACC::col_local(cs, lane), col = colw + cl;
@@ -429,20 +436,58 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
             else *reinterpret_cast<uint2*>(crow + col) = o2;
             if (EPI == CDM_EPI_QKV_PACK && region == 1) {
                 const float a = bf16lo(o2.x), b = bf16hi(o2.x), c = bf16lo(o2.y), d = bf16hi(o2.y);
-                rsq += a * a + b * b + c * c + d * d;
+                rsq[cs / (CS / 2)] += a * a + b * b + c * c + d * d;
             }
         }
         if (EPI == CDM_EPI_QKV_PACK && region == 1) {      // the row's channels are spread over the four quarter-waves
-            rsq += __shfl_xor(rsq, 16, 64);
-            rsq += __shfl_xor(rsq, 32, 64);
-            ksq = fmaxf(ksq, rsq);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                rsq[h] += __shfl_xor(rsq[h], 16, 64);
+                rsq[h] += __shfl_xor(rsq[h], 32, 64);
+            }
+            if (hd64) { ksq[0] = fmaxf(ksq[0], rsq[0]); ksq[1] = fmaxf(ksq[1], rsq[1]); }
+            else ksq[0] = fmaxf(ksq[0], rsq[0] + rsq[1]);
         }
     }
     if (EPI == CDM_EPI_QKV_PACK && region != 0) {
-        // the wave's 64 x 128 piece is one (64-key tile, head) image; staged row r = key r of the tile
+        // the wave's 64 x 128 piece is one (64-key tile, head) image, or two of heads with 64 channels; staged row r = key r
+        // of the tile
         static_assert(EPI != CDM_EPI_QKV_PACK || (ROWS == 64 && CS == 8), "QKV_PACK needs the 64 x 128 wave piece");
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the wave's own staging writes have landed
         const int key_tile = row0 >> 6;
+        if (hd64) {
+            const int head0 = (colw - (region == 1 ? p.d_q : p.d_q + p.d_kv)) >> 6;
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int64_t tile_at = (int64_t)(head0 + hh) * p.n_key_tiles + key_tile;
+                if (region == 1) {      // K image, chunk-major [8 chunks of 8 channels][64 keys][16 bytes]
+                    char* dst = p.kp + tile_at * (64 * 64 * 2);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+                        *reinterpret_cast<uint4*>(dst + (c * 64 + lane) * 16) =
+                            *reinterpret_cast<const uint4*>(stage + lane * kStagePitch + (8 * hh + c) * 16);
+                    float kq = ksq[hh];
+#pragma unroll
+                    for (int off = 1; off < 16; off <<= 1) kq = fmaxf(kq, __shfl_xor(kq, off, 64));
+                    if (lane == 0) p.kmax[tile_at] = sqrtf(kq);
+                } else {                // V^T image [8 chunks][64 channel rows][8 keys], keys of a chunk as below
+                    char* dst = p.vp + tile_at * (64 * 64 * 2);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        uint32_t w[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int key = 32 * (c >> 2) + 4 * (c & 3) + 16 * (e >> 1) + 2 * (e & 1);
+                            const uint32_t lo = *reinterpret_cast<const uint16_t*>(stage + key * kStagePitch + (64 * hh + lane) * 2);
+                            const uint32_t hi = *reinterpret_cast<const uint16_t*>(stage + (key + 1) * kStagePitch + (64 * hh + lane) * 2);
+                            w[e] = lo | (hi << 16);
+                        }
+                        *reinterpret_cast<uint4*>(dst + (c * 64 + lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                }
+            }
+            return;
+        }
         const int head = (colw - (region == 1 ? p.d_q : p.d_q + p.d_kv)) >> 7;
         const int64_t img = ((int64_t)head * p.n_key_tiles + key_tile) * (64 * 128 * 2);
         if (region == 1) {
@@ -452,9 +497,10 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& t, ACC
             for (int c = 0; c < 16; ++c)
                 *reinterpret_cast<uint4*>(dst + (c * 64 + lane) * 16) =
                     *reinterpret_cast<const uint4*>(stage + lane * kStagePitch + c * 16);
+            float kq = ksq[0];
 #pragma unroll
-            for (int off = 1; off < 16; off <<= 1) ksq = fmaxf(ksq, __shfl_xor(ksq, off, 64));
-            if (lane == 0) p.kmax[(int64_t)head * p.n_key_tiles + key_tile] = sqrtf(ksq);
+            for (int off = 1; off < 16; off <<= 1) kq = fmaxf(kq, __shfl_xor(kq, off, 64));
+            if (lane == 0) p.kmax[(int64_t)head * p.n_key_tiles + key_tile] = sqrtf(kq);
         } else {
             // V^T image [8 chunks][128 channel rows][8 keys]; chunk c = 4 s + g lists keys 32 s + 4 g + {0..3} and
             // 32 s + 16 + 4 g + {0..3} (the order in which a lane of the attention kernel holds its probabilities)
@@ -920,9 +966,13 @@ int32_t qkv_pack(const char* who, const void* A, int64_t lda, const float* sa, c
                  int64_t K, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, const float* cos, const float* sin,
                  const cdm_qk_norm* qk_norm, void* workspace, int64_t workspace_bytes, void* stream) {
     CDM_REQUIRE(seg_start && seg_len && workspace, CDM_ERR_BAD_ARG, "%s: null pointer", who);
-    CDM_REQUIRE(head_dim == 128, CDM_ERR_UNSUPPORTED, "%s: head_dim=%d (the fused images need 128)", who, head_dim);
+    CDM_REQUIRE(head_dim == 128 || head_dim == 64, CDM_ERR_UNSUPPORTED, "%s: head_dim=%d (the fused images need 64 or 128)", who,
+                head_dim);
     CDM_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && n_heads <= 65535, CDM_ERR_BAD_SHAPE,
                 "%s: n_kv_heads=%d must divide n_heads=%d", who, n_kv_heads, n_heads);
+    // a wave writes the images of 128 consecutive columns: the Q | K | V boundaries must not cut through such a piece
+    CDM_REQUIRE(head_dim == 128 || (n_heads % 2 == 0 && n_kv_heads % 2 == 0), CDM_ERR_UNSUPPORTED,
+                "%s: head_dim 64 needs even head counts (n_heads=%d, n_kv_heads=%d)", who, n_heads, n_kv_heads);
     CDM_REQUIRE((cos == nullptr) == (sin == nullptr), CDM_ERR_BAD_ARG, "%s: cos and sin must be given together", who);
     CDM_REQUIRE(cdm_aligned16(cos) && cdm_aligned16(sin) && cdm_aligned16(workspace), CDM_ERR_BAD_ALIGN,
                 "%s: rotary tables and workspace must be 16-byte aligned", who);

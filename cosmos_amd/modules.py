@@ -96,8 +96,8 @@ class DMAttnProcessor:
     the attention kernel and to Q when that kernel loads it - no extra pass over memory), "gemm_epilogue" (on the
     fp32 accumulators of the QKV GEMM) or "streaming" (the in-place kernel after a plain QKV GEMM).
     ``fuse_kv_pack`` (with "in_attention"): the QKV GEMM writes K and V straight into the attention kernel's tile
-    images instead of rows that a second kernel re-tiles; taken where the layout allows it (head_dim 128, every
-    token segment starting on a multiple of 64), the two-kernel form otherwise.
+    images instead of rows that a second kernel re-tiles; taken where the layout allows it (head_dim 128, or 64 with
+    even head counts; every token segment starting on a multiple of 64), the two-kernel form otherwise.
     """
 
     def __init__(self, rope: str = "in_attention", fuse_kv_pack: bool = True):
@@ -158,7 +158,8 @@ class DMAttnProcessor:
                          rope_cols=d + dkv, head_dim=attn.head_dim)
             ops.attention(q, k, v, attn.n_heads, attn.head_dim, out=o, workspace=wsb, **mask_kw)
         elif (self.rope == "in_attention" and self.fuse_kv_pack
-              and ops.qkv_pack_applies([(s0, ln) for (s0, ln, _, _) in modality_segments], attn.head_dim)):
+              and ops.qkv_pack_applies([(s0, ln) for (s0, ln, _, _) in modality_segments], attn.head_dim, attn.n_heads,
+                                       attn.n_kv_heads)):
             if wsb is None:
                 wsb = torch.empty((ops.attn_workspace_total_bytes(n, attn.n_heads, attn.n_kv_heads, attn.head_dim),),
                                   dtype=torch.uint8, device=x.device)

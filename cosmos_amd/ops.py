@@ -377,15 +377,16 @@ def gemm_qkv_pack(a: torch.Tensor, sa: Optional[torch.Tensor], ws: Sequence[torc
         _lib.check(rc, "cdm_grouped_gemm_qkv_pack_fp8")
 
 
-def qkv_pack_applies(segments: Sequence[Tuple[int, int]], head_dim: int) -> bool:
-    """Whether ``gemm_qkv_pack`` accepts this token layout: head_dim 128, segments tiling [0, n) in order, each
-    starting on a multiple of 64 tokens (a 64-key tile image is written by one wave from one weight set)."""
+def qkv_pack_applies(segments: Sequence[Tuple[int, int]], head_dim: int, n_heads: int = 2, n_kv_heads: int = 2) -> bool:
+    """Whether ``gemm_qkv_pack`` accepts this layout: head_dim 128, or 64 with even head counts (a wave writes the
+    images of 128 consecutive columns), segments tiling [0, n) in order, each starting on a multiple of 64 tokens (a
+    64-key tile image is written by one wave from one weight set)."""
     pos = 0
     for s, l in segments:
         if int(s) != pos or pos % 64:
             return False
         pos += int(l)
-    return head_dim == 128 and pos > 0
+    return pos > 0 and (head_dim == 128 or (head_dim == 64 and n_heads % 2 == 0 and n_kv_heads % 2 == 0))
 
 
 # ----------------------------------------------------------------------------- RoPE / attention

@@ -329,7 +329,8 @@ int32_t cdm_set_variant(const char* op, int32_t variant);
  * to the fp32 accumulators ahead of the rotation, segment g of the projection using row g of qk_norm->k_weight
  * (qk_norm->n_seg = n_seg, qk_norm->seg_end[g] = seg_start[g] + seg_len[g]); the Q rows leave un-normalised -
  * cdm_attn_fwd_packed_bf16 normalises and rotates them at load when given the same descriptor.
- * Restrictions: head_dim 128; the segments tile [0, n_tokens) in order and each starts on a multiple of 64 tokens
+ * Restrictions: head_dim 128, or 64 with even n_heads and n_kv_heads (a wave writes the images of 128 consecutive
+ * columns); the segments tile [0, n_tokens) in order and each starts on a multiple of 64 tokens
  * (CDM_ERR_UNSUPPORTED otherwise - callers fall back to the GEMM + cdm_attn_pack_kv_bf16 pair).
  */
 int32_t cdm_grouped_gemm_qkv_pack_bf16(const void* A, int64_t lda, const void* const* W, int64_t ldw, void* Q,

@@ -139,7 +139,7 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.cdm_quant_rows_from_parts_e4m3(fake, 128, fake, 4, 4, fake, fake, 0, 128, None) in (_lib.OK, _lib.ERR_NO_DEVICE)
     # the workspace holds K/V heads only
     assert lib.cdm_attn_workspace_bytes(100, 2, 64) * 3 == lib.cdm_attn_workspace_bytes(100, 6, 64)
-    # QKV projection with fused tile images: head_dim 128 only, segments tile the sequence on 64-token boundaries,
+    # QKV projection with fused tile images: head_dim 128 (or 64 with even head counts), segments tile the sequence on 64-token boundaries,
     # the workspace must hold the images, and the general GEMM entry points refuse its epilogue code
     W = (C.c_void_p * 2)(fake, fake)
 
@@ -147,7 +147,9 @@ def test_bad_arguments_are_rejected_on_the_host():
         st, ln = (C.c_int64 * len(starts))(*starts), (C.c_int64 * len(lens))(*lens)
         return lib.cdm_grouped_gemm_qkv_pack_bf16(fake, 256, W, 256, fake, H * hd, st, ln, len(starts), 256, H, Hkv, hd, None, None,
                                                   qkn, fake, ws, None)
-    assert qp([0], [100], hd=64) == _lib.ERR_UNSUPPORTED
+    assert qp([0], [100], hd=32) == _lib.ERR_UNSUPPORTED
+    assert qp([0], [100], hd=64, H=3, Hkv=3) == _lib.ERR_UNSUPPORTED and "even head counts" in _lib.last_error()
+    assert qp([0], [100], hd=64) in (_lib.OK, _lib.ERR_NO_DEVICE, _lib.ERR_LAUNCH)      # accepted: fails only for want of a device
     assert qp([0, 100], [100, 28]) == _lib.ERR_UNSUPPORTED and "multiple of 64" in _lib.last_error()
     assert qp([0, 128], [64, 64]) == _lib.ERR_UNSUPPORTED           # a gap between the segments
     assert qp([0], [100], ws=1024) == _lib.ERR_BAD_ARG and "workspace" in _lib.last_error()

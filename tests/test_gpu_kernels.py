@@ -275,25 +275,27 @@ def test_gemm_gate_residual_fp32_stream(M, N, K, gated, fp8, variant, request):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("n,H,Hkv,K,rope,split,qkn", [(256, 2, 2, 256, False, 0, False), (1000, 4, 2, 512, True, 0, False),
-                                                     (800, 2, 1, 256, True, 320, False), (4100, 3, 3, 256, False, 1024, False),
-                                                     (64, 1, 1, 256, True, 0, False), (1000, 4, 2, 512, True, 0, True),
-                                                     (800, 2, 1, 256, True, 320, True), (300, 2, 2, 256, False, 128, True)])
-def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, qkn, fp8):
+@pytest.mark.parametrize("n,H,Hkv,K,rope,split,qkn,hd", [(256, 2, 2, 256, False, 0, False, 128), (1000, 4, 2, 512, True, 0, False, 128),
+                                                        (800, 2, 1, 256, True, 320, False, 128), (4100, 3, 3, 256, False, 1024, False, 128),
+                                                        (64, 1, 1, 256, True, 0, False, 128), (1000, 4, 2, 512, True, 0, True, 128),
+                                                        (800, 2, 1, 256, True, 320, True, 128), (300, 2, 2, 256, False, 128, True, 128),
+                                                        (256, 2, 2, 256, False, 0, False, 64), (1000, 8, 2, 512, True, 0, False, 64),
+                                                        (800, 6, 2, 256, True, 320, True, 64), (300, 4, 4, 256, False, 128, True, 64)])
+def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, qkn, hd, fp8):
     """The QKV GEMM that writes K and V as the attention kernel's tile images, against the plain GEMM followed by the
     re-tiling kernel: same Q rows, same V image and (without rotation or norm) the same K image bit for bit, the same
     key-norm bounds to fp32 rounding; with rotation or the per-head RMSNorm K carries one rounding less (both act on the
     fp32 accumulators), so the images agree to a bf16 ulp and the attention outputs to 1e-2.
     Ragged last tiles (1000, 800, 4100, 300 tokens), grouped K / V heads, two weight sets (and two norm weight rows)
-    split on a tile boundary; with the norm the attention output is also checked against the oracle."""
-    hd = 128
+    split on a tile boundary; with the norm the attention output is also checked against the oracle.  head_dim 64: a
+    wave's 128 columns are two heads (two images, two norms, two key-norm bounds); odd head counts are refused."""
     g = gen(n + 7 * H + K)
     d, dkv = H * hd, Hkv * hd
     a, _ = rand_bf16((n, K), g)
     segs = [(0, n)] if not split else [(0, split), (split, n - split)]
     ws = [rand_bf16((d + 2 * dkv, K), g, 0.05)[0] for _ in segs]
     pos, _ = rotary.build_positions(0, (1, 1, n))
-    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48), device=dev()) if rope else (None, None)
+    cos, sin = rotary.rotary_tables(pos, hd, (32, 48, 48) if hd == 128 else (16, 24, 24), device=dev()) if rope else (None, None)
     norm = None
     if qkn:
         qw = 1.0 + 0.3 * torch.randn(len(segs), hd, generator=g)
@@ -328,7 +330,8 @@ def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, qkn, fp8):
         assert torch.allclose(km, km_ref, rtol=1e-2)
     o = ops.attention_packed(q_out, img, H, hd, None, cos, sin, norm, None, 0, Hkv)
     o_ref = ops.attention_packed(q, img_ref, H, hd, None, cos, sin, norm, None, 0, Hkv)
-    assert_close(o, o_ref, 0.9999, 1e-2, f"attention on fused images n={n} fp8={fp8} qkn={qkn}")
+    # (the two paths round K at different points; heads of 64 channels with the norm and e4m3 operands spread furthest)
+    assert_close(o, o_ref, 0.9999, 2e-2 if (hd == 64 and qkn) else 1e-2, f"attention on fused images n={n} hd={hd} fp8={fp8} qkn={qkn}")
     if qkn:      # against the oracle, from the projected rows the kernels saw (bf16 Q / K / V of the plain GEMM)
         qr, kr_, vr = q.float().cpu().view(n, H, hd), k.float().cpu().view(n, Hkv, hd), v.float().cpu().view(n, Hkv, hd)
         qn_, kn_ = torch.empty_like(qr), torch.empty_like(kr_)
@@ -341,6 +344,7 @@ def test_gemm_qkv_pack(n, H, Hkv, K, rope, split, qkn, fp8):
         want = O.attention(qn_, kn_.repeat_interleave(rep, dim=1), vr.repeat_interleave(rep, dim=1))
         assert_close(o, want.reshape(n, d), 0.9999, 1e-2, f"fused images with K-norm vs oracle n={n} fp8={fp8}")
     # layouts the fused form does not take are refused, not mis-tiled
+    assert ops.qkv_pack_applies(segs, hd, H, Hkv) and not ops.qkv_pack_applies(segs, 64, 3, 3)
     if n > 100:
         with pytest.raises(RuntimeError):
             ops.gemm_qkv_pack(a if not fp8 else aq, sa if fp8 else None, [ws[0]] * 2 if not fp8 else [wq[0][0]] * 2,
