@@ -56,13 +56,18 @@ __global__ __launch_bounds__(kThreads) void adaln_rmsnorm_kernel(
     for (int c = 0; c < MAXC; ++c) {
         const int idx = c * kThreads + tid;
         if (idx < nchunk) {
+            // 16-byte loads: a workgroup walks over a few rows only (see the grid), so this set-up must stay cheap
             float wv[8];
             unpack8(w[idx], wv);
+            float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0, h0 = s0, h1 = s0;
+            if (scale) { s0 = reinterpret_cast<const float4*>(scale)[2 * idx]; s1 = reinterpret_cast<const float4*>(scale)[2 * idx + 1]; }
+            if (shift) { h0 = reinterpret_cast<const float4*>(shift)[2 * idx]; h1 = reinterpret_cast<const float4*>(shift)[2 * idx + 1]; }
+            const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            const float sh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float sc = scale ? scale[idx * 8 + i] : 0.0f;
-                a[c][i] = wv[i] * (1.0f + sc);
-                b[c][i] = shift ? shift[idx * 8 + i] : 0.0f;
+                a[c][i] = wv[i] * (1.0f + sc[i]);
+                b[c][i] = sh[i];
             }
         } else {
 #pragma unroll
@@ -239,7 +244,10 @@ __global__ __launch_bounds__(kThreads) void quant_rows_parts_kernel(const bf16_t
 template <bool QUANT, bool XF32>
 int32_t launch_norm(const void* x, const void* w, const float* shift, const float* scale, void* y, float* s_tok,
                     int64_t n_tokens, int64_t d, float eps, hipStream_t st) {
-    const int64_t max_blocks = 256 * 8;
+    // 64 workgroups per CU's worth of rows in flight: at 56 k rows a workgroup walks over three or four rows.  Measured in
+    // the 56,832 x 4096 stack (fp32 rows in, bf16 out): 2048 workgroups 5.37 TB/s, 4096 5.53, 8192 5.63, 16384 5.75, 32768
+    // 5.52, one row each 5.04 (the per-channel vectors are then loaded as often as the rows)
+    const int64_t max_blocks = 256 * 64;
     const int grid = (int)(n_tokens < max_blocks ? n_tokens : max_blocks);
     const int chunks = (int)((d / 8 + kThreads - 1) / kThreads);
 #define CDM_NORM_LAUNCH(C)                                                                                  \
@@ -252,13 +260,14 @@ int32_t launch_norm(const void* x, const void* w, const float* shift, const floa
     return cdm_check_launch("adaln_rmsnorm");
 }
 
-int32_t check_norm_args(const void* x, const void* w, const void* y, int64_t n_tokens, int64_t d) {
+int32_t check_norm_args(const void* x, const void* w, const void* y, int64_t n_tokens, int64_t d, const float* shift,
+                        const float* scale) {
     CDM_REQUIRE(x && w && y, CDM_ERR_BAD_ARG, "adaln_rmsnorm: null pointer");
     CDM_REQUIRE(n_tokens >= 0 && d > 0, CDM_ERR_BAD_ARG, "adaln_rmsnorm: negative size");
     CDM_REQUIRE(d % 8 == 0 && d <= 8192, CDM_ERR_BAD_SHAPE, "adaln_rmsnorm: d=%lld must be a multiple of 8 and <= 8192",
                 (long long)d);
-    CDM_REQUIRE(cdm_aligned16(x) && cdm_aligned16(w) && cdm_aligned16(y), CDM_ERR_BAD_ALIGN,
-                "adaln_rmsnorm: pointers must be 16-byte aligned");
+    CDM_REQUIRE(cdm_aligned16(x) && cdm_aligned16(w) && cdm_aligned16(y) && cdm_aligned16(shift) && cdm_aligned16(scale),
+                CDM_ERR_BAD_ALIGN, "adaln_rmsnorm: pointers must be 16-byte aligned");
     return CDM_OK;
 }
 
@@ -266,7 +275,7 @@ int32_t check_norm_args(const void* x, const void* w, const void* y, int64_t n_t
 
 extern "C" int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const float* shift, const float* scale,
                                           void* y, int64_t n_tokens, int64_t d, float eps, void* stream) {
-    int32_t rc = check_norm_args(x, w, y, n_tokens, d);
+    int32_t rc = check_norm_args(x, w, y, n_tokens, d, shift, scale);
     if (rc) return rc;
     if ((rc = cdm_require_device())) return rc;
     if (n_tokens == 0) return CDM_OK;
@@ -275,7 +284,7 @@ extern "C" int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const fl
 
 extern "C" int32_t cdm_adaln_rmsnorm_f32(const float* x, const void* w, const float* shift, const float* scale,
                                          void* y, int64_t n_tokens, int64_t d, float eps, void* stream) {
-    int32_t rc = check_norm_args(x, w, y, n_tokens, d);
+    int32_t rc = check_norm_args(x, w, y, n_tokens, d, shift, scale);
     if (rc) return rc;
     if ((rc = cdm_require_device())) return rc;
     if (n_tokens == 0) return CDM_OK;
@@ -285,7 +294,7 @@ extern "C" int32_t cdm_adaln_rmsnorm_f32(const float* x, const void* w, const fl
 extern "C" int32_t cdm_adaln_rmsnorm_quant_e4m3(const void* x, const void* w, const float* shift,
                                                 const float* scale, void* yq, float* s_tok, int64_t n_tokens,
                                                 int64_t d, float eps, void* stream) {
-    int32_t rc = check_norm_args(x, w, yq, n_tokens, d);
+    int32_t rc = check_norm_args(x, w, yq, n_tokens, d, shift, scale);
     if (rc) return rc;
     CDM_REQUIRE(s_tok, CDM_ERR_BAD_ARG, "adaln_rmsnorm_quant: null s_tok");
     if ((rc = cdm_require_device())) return rc;
@@ -296,7 +305,7 @@ extern "C" int32_t cdm_adaln_rmsnorm_quant_e4m3(const void* x, const void* w, co
 extern "C" int32_t cdm_adaln_rmsnorm_f32_quant_e4m3(const float* x, const void* w, const float* shift,
                                                     const float* scale, void* yq, float* s_tok, int64_t n_tokens,
                                                     int64_t d, float eps, void* stream) {
-    int32_t rc = check_norm_args(x, w, yq, n_tokens, d);
+    int32_t rc = check_norm_args(x, w, yq, n_tokens, d, shift, scale);
     if (rc) return rc;
     CDM_REQUIRE(s_tok, CDM_ERR_BAD_ARG, "adaln_rmsnorm_quant: null s_tok");
     if ((rc = cdm_require_device())) return rc;
@@ -315,7 +324,9 @@ extern "C" int32_t cdm_quant_rows_e4m3(const void* a, int64_t lda, void* q, floa
     int32_t rc = cdm_require_device();
     if (rc) return rc;
     if (rows == 0) return CDM_OK;
-    const int64_t max_blocks = 256 * 8;
+    // one row per workgroup: nothing is set up per workgroup, and rows then stream in address order (56,832 x 4096 and
+    // x 16384 bf16 rows: 6.0 TB/s against 5.2 with 2048 workgroups walking over the rows, 5.8 with 8192)
+    const int64_t max_blocks = (1ll << 31) - 1;
     const int grid = (int)(rows < max_blocks ? rows : max_blocks);
     quant_rows_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>((const bf16_t*)a, lda, (uint8_t*)q, s, rows,
                                                                   (int)cols);
@@ -336,7 +347,9 @@ extern "C" int32_t cdm_quant_rows_from_parts_e4m3(const void* a, int64_t lda, co
     int32_t rc = cdm_require_device();
     if (rc) return rc;
     if (rows == 0) return CDM_OK;
-    const int64_t max_blocks = 256 * 8;
+    // one row per workgroup: nothing is set up per workgroup, and rows then stream in address order (56,832 x 4096 and
+    // x 16384 bf16 rows: 6.0 TB/s against 5.2 with 2048 workgroups walking over the rows, 5.8 with 8192)
+    const int64_t max_blocks = (1ll << 31) - 1;
     const int grid = (int)(rows < max_blocks ? rows : max_blocks);
     quant_rows_parts_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>((const bf16_t*)a, lda, parts, ldp, (int)n_parts,
                                                                         (uint8_t*)q, s, rows, (int)cols);
