@@ -69,7 +69,8 @@ int32_t cdm_device_count(void);
  * transformers Qwen3VLTextRMSNorm.forward, models/qwen3_vl/modeling_qwen3_vl.py:400-405).
  *   y[i,j] = x[i,j] * rsqrt(mean_j x[i,:]^2 + eps) * w[j] * (1 + scale[j]) + shift[j]
  * x, y: [n_tokens, d] bf16 (y may alias x); w: [d] bf16; shift, scale: [d] fp32, either may be
- * null (plain RMSNorm of the AR branch).  d % 8 == 0, d <= 8192.
+ * null (plain RMSNorm of the AR branch).  d % 8 == 0, d <= 8192; all pointers 16-byte aligned (shift and scale too:
+ * slices of a [6 d] modulation row are, since d % 8 == 0).
  */
 int32_t cdm_adaln_rmsnorm_bf16(const void* x, const void* w, const float* shift, const float* scale,
                                void* y, int64_t n_tokens, int64_t d, float eps, void* stream);

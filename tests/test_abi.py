@@ -65,6 +65,7 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert "null" in _lib.last_error()
     assert lib.cdm_adaln_rmsnorm_bf16(fake, fake, None, None, fake, 4, 60, 1e-6, None) == _lib.ERR_BAD_SHAPE
     assert lib.cdm_adaln_rmsnorm_bf16(fake + 2, fake, None, None, fake, 4, 64, 1e-6, None) == _lib.ERR_BAD_ALIGN
+    assert lib.cdm_adaln_rmsnorm_bf16(fake, fake, fake + 4, None, fake, 4, 64, 1e-6, None) == _lib.ERR_BAD_ALIGN      # shift
     g = lambda **kw: lib.cdm_gemm_bf16(kw.get("A", fake), kw.get("lda", 128), fake, 128, kw.get("W2", None), fake, 256, 8, 256,
                                        kw.get("K", 128), kw.get("epi", 0), kw.get("R", None), 256, None, None, None,
                                        kw.get("rope_cols", 0), kw.get("hd", 0), None)
